@@ -44,55 +44,56 @@ class CacheGroupLayout:
 
 class CacheLayout:
     def __init__(self, groups: list, layer_group: dict, states: dict):
+        # (a key is a layer's index, or what the schedule gives a run of a layer that runs several times)
         self.groups = groups            # [CacheGroupLayout]
-        self.layer_group = layer_group  # layer index -> group index (layers that own pools)
-        self.states = states            # layer index -> StateSpec
+        self.layer_group = layer_group  # key -> group index (runs that own pools)
+        self.states = states            # key -> StateSpec
 
     @classmethod
     def from_blocks(cls, blocks, schedule) -> "CacheLayout":
         # A run of a layer either owns its cache or reads the one another run has written earlier in the
-        # same pass.  Two owning runs of one layer would write the same pages twice, and what a later step
+        # same pass.  What a run owns is kept under a key: the layer's index, or the key the schedule gives
+        # the run (a layer that runs several times with the same weights then has pages and state for every
+        # run).  Two owning runs under one key would write the same pages twice, and what a later step
         # reads there would depend on how the tokens were cut into steps: refused.
         def spec_of(index):
             mixer = getattr(blocks[index], "mixer", None)
             return (mixer.cache_spec(), mixer.state_spec()) if mixer is not None else (None, None)
 
-        written: set = set()
+        written: dict = {}           # key -> the layer whose run owns it
         for at, e in enumerate(schedule):
             kv, state = spec_of(e.layer)
             if e.cache_from is None:
-                if e.layer in written and (kv is not None or state is not None):
-                    raise ConfigError(f"the schedule runs layer {e.layer} twice with a cache of its own; the second run "
-                                      f"can read what the first wrote (cache_from={e.layer})")
-                written.add(e.layer)
+                key = e.layer if e.cache_key is None else e.cache_key
+                if key in written and (kv is not None or state is not None):
+                    raise ConfigError(f"the schedule runs layer {e.layer} twice with one cache; the second run can read "
+                                      f"what the first wrote (cache_from={key}) or keep a cache of its own (cache_key)")
+                written[key] = e.layer
             else:
                 if e.cache_from not in written:
                     raise ConfigError(f"run {at} of the schedule reads the cache of layer {e.cache_from}, which no "
                                       "earlier run of the pass has written")
                 if state is not None:
                     raise ConfigError(f"layer {e.layer} keeps a state of its own and cannot read another layer's cache")
-                if spec_of(e.cache_from)[0] != kv:
+                if spec_of(written[e.cache_from])[0] != kv:
                     raise ConfigError(f"layer {e.layer} reads the cache of layer {e.cache_from}, whose keys and values "
                                       "have another shape or window")
-        owners = sorted(written)
         groups: list = []
         layer_group: dict = {}
         states: dict = {}
-        for index in owners:
-            mixer = getattr(blocks[index], "mixer", None)
-            spec = mixer.cache_spec() if mixer is not None else None
+        for key in sorted(written):
+            spec, state = spec_of(written[key])
             if spec is not None:
                 for g, group in enumerate(groups):
                     if group.spec == spec:
-                        group.layers.append(index)
-                        layer_group[index] = g
+                        group.layers.append(key)
+                        layer_group[key] = g
                         break
                 else:
-                    groups.append(CacheGroupLayout(spec, [index]))
-                    layer_group[index] = len(groups) - 1
-            state = mixer.state_spec() if mixer is not None else None
+                    groups.append(CacheGroupLayout(spec, [key]))
+                    layer_group[key] = len(groups) - 1
             if state is not None:
-                states[index] = state
+                states[key] = state
         return cls(groups, layer_group, states)
 
     def bytes_per_token(self, element_size: int) -> int:

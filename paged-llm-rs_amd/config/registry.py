@@ -10,6 +10,7 @@ from pathlib import Path
 
 from ..errors import ConfigError, UnsupportedError
 from .lefavik import LefavikConfig
+from .mukenex import MukenexConfig
 from .papivik import PapivikConfig
 from .qwen3 import Qwen3Config, read_json
 
@@ -66,3 +67,4 @@ def load_config(source):
 register_architecture("Qwen3ForCausalLM", Qwen3Config, model_type="qwen3")
 register_architecture("Papivik", PapivikConfig, model_type="papivik")
 register_architecture("Lefavik", LefavikConfig, model_type="lefavik")
+register_architecture("Mukenex", MukenexConfig, model_type="mukenex")

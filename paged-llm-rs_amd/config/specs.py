@@ -17,6 +17,7 @@ class NormSpec:
     """A normalisation over the last axis."""
     kind: str = "rms_norm"
     eps: float = 1e-6
+    gain_offset: float = 0.0                # the stored gain plus this is the gain (1.0: gains stored around zero)
 
 
 @dataclass(frozen=True)
@@ -63,6 +64,7 @@ class LayerSpec:
     norm: Any = None
     weight_prefix: str = ""
     names: Optional[dict] = None            # other tensor-name parts for the block's members (norm1, mixer, norm2, feed_forward)
+    stream_copies: Optional[int] = None     # for an arrangement over several copies of the stream: how many
 
 
 @dataclass(frozen=True)
@@ -72,6 +74,10 @@ class ScheduleEntry:
     writing its own."""
     layer: int
     cache_from: Optional[int] = None
+    # A layer that runs several times with the same weights keeps pages and state of its own for every run:
+    # runs with different ``cache_key`` (any numbers; None is the layer's own index) share nothing.  ``cache_from``
+    # names the key that is read.
+    cache_key: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -191,6 +197,11 @@ class SinkAttentionSpec:
     slope_span: float = 8.0
     window: Optional[int] = None            # keys j with i - window < j <= i; None: all keys up to i
     sink: Optional[str] = "zero"            # "zero": a sink of score 0; "learned": one a head (tensor ``sink``); None
+    # "window": as above.  "block": positions are cut into blocks of ``window`` counted from position 0 of the
+    # request, and a query sees the keys of its own block up to itself.
+    mask: str = "window"
+    qk_gain: bool = False                   # the unit q and k times a gain over the head (tensors ``q.norm``, ``k.norm``)
+    qkv_bias: bool = False                  # q, k and v projections carry a bias each (``q.b``, ``k.b``, ``v.b``)
 
 
 @dataclass(frozen=True)
@@ -206,10 +217,25 @@ class LatentAttentionSpec:
     kv_rank: int = 0
     rotary_turned: int = 0                  # how many values of the rotated part turn (pairs 2i, 2i + 1)
     rotary_base: float = 10000.0
-    max_positions: int = 0                  # rows of the rotation's tables
+    max_positions: int = 0                  # rows of the rotation's tables; 0: no tables, angles worked out in the kernel
     scale: Optional[float] = None           # None = 1/sqrt(head_dim + rotary_dim)
     norm_eps: float = 1e-6                  # of the norm on the small vector
     sink: Optional[str] = "learned"         # as in SinkAttentionSpec
     gated: bool = True                      # a head's read-out times sigmoid(gate projection of the layer's input)
+    gate_each: str = "head"                 # one gate a "head" (tensor ``g`` [heads, width]) or an "element" ([heads * value_dim, width])
     window: Optional[int] = None
     borrows: bool = False                   # no projection onto the small vector: the schedule names the layer whose pages are read
+
+
+# ---- several copies of the stream, experts chosen by a table ----------------------------------------
+
+@dataclass(frozen=True)
+class TableExpertsSpec:
+    """``experts`` small gated feed-forwards, down(act(gate x) * (up x)), of which a token uses the ``top`` that
+    a table names for its id (tensor ``table`` [vocabulary, top]); each of them counts 1/top."""
+    kind: str = "table_experts"
+    experts: int = 0
+    top: int = 0
+    intermediate_size: int = 0
+    vocab_size: int = 0
+    activation: str = "silu"

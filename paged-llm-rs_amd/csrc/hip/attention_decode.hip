@@ -255,7 +255,7 @@ paged_attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t
     const int at8 = min(dl * 8, d - 8);
 
     // the stretch of keys of this split, in whole rounds of the workgroup
-    const int first = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+    const int first = pl_first_visible(pos, window);
     const int limit = fuse.mode == 2 ? pos : pos + 1;   // the token's own key is not in the cache yet
     const int total = max(limit - first, 0);
     // ceil(total / splits): the high half of (total + splits - 1) * ceil(2^32 / splits), exact below 2^32 / splits
@@ -747,7 +747,7 @@ extern "C" int pl_paged_attention_decode(const void* q, int q_stride, void* out,
                                          int rot, const float* sinks, const float* slopes, hipStream_t stream) {
     PL_REQUIRE(d > 0 && d <= 256 && d % 16 == 0, "decode attention: head size %d, which has to be a multiple of 16 up to 256", d);
     PL_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "decode attention: %d query heads over %d key heads", nq, nkv);
-    PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && window >= 0 && splits >= 1 && splits <= AD_MAX_SPLITS,
+    PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && splits >= 1 && splits <= AD_MAX_SPLITS,
                "decode attention: block size %d, %d blocks a row, query stride %d, window %d, %d splits", block_size,
                max_blocks, q_stride, window, splits);
     PL_REQUIRE(splits == 1 || (part_acc && part_ml), "decode attention: %d splits without a workspace", splits);

@@ -39,7 +39,7 @@ paged_attention_plain_kernel(const T* __restrict__ q, int q_stride, T* __restric
     __syncthreads();
 
     const int* table = block_table + static_cast<size_t>(seq_of[t]) * max_blocks;
-    const int first = (window > 0 && pos + 1 > window) ? pos + 1 - window : 0;
+    const int first = pl_first_visible(pos, window);
     const float slope = slopes != nullptr ? slopes[h] : 0.f;
 
     float m = -INFINITY, l = 0.f;
@@ -107,7 +107,7 @@ extern "C" int pl_paged_attention_plain(const void* q, int q_stride, void* out, 
                                         const float* sinks, const float* slopes, hipStream_t stream) {
     PL_REQUIRE(d > 0 && d <= PL_MAX_HEAD_DIM, "attention: head size %d, which has to be between 1 and %d", d, PL_MAX_HEAD_DIM);
     PL_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "attention: %d query heads over %d key heads", nq, nkv);
-    PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && window >= 0,
+    PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d,
                "attention: block size %d, %d blocks a row, query stride %d, window %d", block_size, max_blocks, q_stride, window);
     PL_REQUIRE(nq <= 65535, "attention: %d query heads are more than one launch covers", nq);
     if (n <= 0) return 0;

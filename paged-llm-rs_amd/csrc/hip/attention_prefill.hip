@@ -279,7 +279,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     float m = -INFINITY, lsum = 0.f;
 
     const int last_pos = GR ? start + q0 : start + min(q0 + BM, count) - 1;   // the last key any query of the tile sees
-    const int first_pos = (window > 0 && start + q0 + 1 > window) ? start + q0 + 1 - window : 0;
+    const int first_pos = pl_first_visible(start + q0, window);
     const int* table = block_table + static_cast<size_t>(seq) * max_blocks;
     const size_t row_stride = static_cast<size_t>(nkv) * d;
     const size_t head_off = static_cast<size_t>(kvh) * d;
@@ -616,7 +616,8 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     auto soften = [&](int k0, bool masked) {
         float mx = -INFINITY;
         // Key k0 + c + 4*h, c a constant of the register, is seen by this lane's query iff c <= reach
-        // (and c > reach - window); it stands reach - c positions before the query.
+        // (and c > reach - seen, seen the keys from the first one the query sees to its own); it stands
+        // reach - c positions before the query.
         const int reach = q_pos - k0 - 32 * kt0 - 4 * h;
         if (tilted) {
             const float from = -tilt * static_cast<float>(reach);
@@ -627,7 +628,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                     s[kt][r] += fmaf(tilt, static_cast<float>(32 * kt + 8 * (r >> 2) + (r & 3)), from);
         }
         if (masked) {
-            const int behind = window > 0 ? reach - window : -(1 << 30);
+            const int behind = window != 0 ? reach - (q_pos - pl_first_visible(q_pos, window) + 1) : -(1 << 30);
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -744,7 +745,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
                 for (int w = 0; w < 4; ++w) pb[kt][half].w[w] = 0u;
     };
     no_weights();
-    const int open_end = window > 0 ? k_first : ((start + q0 + 1) / AP_BN) * AP_BN;   // keys below it are seen by all
+    const int open_end = window != 0 ? k_first : ((start + q0 + 1) / AP_BN) * AP_BN;   // keys below it are seen by all
     auto next_tile = [&]() {
         if (k0 != k_first) vbuf_before = vbuf_before + 1 == NVB ? 0 : vbuf_before + 1;
         k0 += AP_BN;
@@ -766,7 +767,7 @@ paged_attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_
     for (; k0 < k_end; next_tile()) {
         // a wave whose queries all stand before this tile, or that has no queries, has nothing to add
         const bool idle = !wave_active || k0 + 32 * kt0 > wave_last ||
-                          (window > 0 && k0 + 32 * (kt0 + KT) - 1 <= wave_first - window);
+                          (window != 0 && k0 + 32 * (kt0 + KT) - 1 < pl_first_visible(wave_first, window));
         if (!ask_late) feed_before();
         multiply(kbuf, vbuf_before, !idle);
         feed_after();
@@ -1043,7 +1044,7 @@ extern "C" int pl_paged_attention_prefill(const void* q, int q_stride, void* out
                "prefill attention: %d splits%s", splits, splits > 1 ? " without a workspace" : "");
     PL_REQUIRE(d > 0 && d <= 256 && d % 16 == 0, "prefill attention: head size %d, which has to be a multiple of 16 up to 256", d);
     PL_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "prefill attention: %d query heads over %d key heads", nq, nkv);
-    PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && window >= 0,
+    PL_REQUIRE(block_size > 0 && max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0,
                "prefill attention: block size %d, %d blocks a row, query stride %d, window %d", block_size, max_blocks,
                q_stride, window);
     PL_REQUIRE((nkv * d) % 8 == 0, "prefill attention: a cache row of %d elements is not read 16 bytes at a time", nkv * d);
@@ -1130,7 +1131,7 @@ extern "C" int pl_paged_attention_grouped(const void* q, int q_stride, void* out
                "grouped attention: %d query heads over %d key heads of %d, pages of %d", nq, nkv, d, block_size);
     PL_REQUIRE(splits >= 1 && splits <= AP_MERGE_MAX && (splits == 1 || (part_acc && part_ml)),
                "grouped attention: %d splits%s", splits, splits > 1 ? " without a workspace" : "");
-    PL_REQUIRE(max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0 && window >= 0,
+    PL_REQUIRE(max_blocks > 0 && q_stride >= nq * d && q_stride % 8 == 0,
                "grouped attention: %d blocks a row, query stride %d, window %d", max_blocks, q_stride, window);
     if (num_seqs <= 0 || max_q_len <= 0) return 0;
     PL_REQUIRE(total_rows >= max_q_len, "grouped attention: %d rows for portions of %d", total_rows, max_q_len);

@@ -111,3 +111,12 @@ int pl_compute_units();
     } while (0)
 
 __host__ __device__ static inline int pl_ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Which keys at or before its own position a query sees, as one number (the attention kernels' `window`):
+// 0 all of them; w > 0 a window, its own key and the w - 1 before it; -c < 0 blocks of c positions counted
+// from position 0 of the request, the keys of the query's own block.  The first key the query at `pos` sees:
+__host__ __device__ static inline int pl_first_visible(int pos, int window) {
+    if (window > 0) return pos + 1 > window ? pos + 1 - window : 0;
+    if (window < 0) return pos - pos % (-window);
+    return 0;
+}

@@ -153,9 +153,11 @@ __global__ __launch_bounds__(64) void latent_prepare_kernel(LatentPrepareArgs a)
     const int pos = a.positions[t];
     if (pos < 0) return;
     const int H = a.H, D = a.D, rot = a.rot, R = a.R, P = a.P;
-    const bool turns = a.turned > 0 && pos < a.table_rows;
-    const float* cs = a.cos + static_cast<size_t>(turns ? pos : 0) * (a.turned / 2);
-    const float* sn = a.sin + static_cast<size_t>(turns ? pos : 0) * (a.turned / 2);
+    // (without tables, `cos` lists the frequencies and the angle is position * frequency, in 32-bit)
+    const bool tables = a.sin != nullptr;
+    const bool turns = a.turned > 0 && (!tables || pos < a.table_rows);
+    const float* cs = a.cos + static_cast<size_t>(turns && tables ? pos : 0) * (a.turned / 2);
+    const float* sn = tables ? a.sin + static_cast<size_t>(turns ? pos : 0) * (a.turned / 2) : nullptr;
     const float* row = a.rows + static_cast<size_t>(t) * a.stride;
     const float* part;        // the rotated part this job turns
     T* dst;                   // where it goes, with the zeros behind it
@@ -186,7 +188,14 @@ __global__ __launch_bounds__(64) void latent_prepare_kernel(LatentPrepareArgs a)
             x = part[e];
             if (turns && e < a.turned) {
                 const int i = e >> 1;
-                x = (e & 1) ? part[e] * cs[i] + part[e - 1] * sn[i] : part[e] * cs[i] - part[e + 1] * sn[i];
+                float c, sn_i;
+                if (tables) {
+                    c = cs[i];
+                    sn_i = sn[i];
+                } else {
+                    sincosf(static_cast<float>(pos) * cs[i], &sn_i, &c);
+                }
+                x = (e & 1) ? part[e] * c + part[e - 1] * sn_i : part[e] * c - part[e + 1] * sn_i;
             }
         }
         dst[e] = from_float<T>(x);
@@ -200,7 +209,7 @@ extern "C" int pl_latent_prepare(const float* rows, int stride, int q_off, int k
                                  int P, hipStream_t stream) {
     PL_REQUIRE(n >= 0 && H > 0 && H < 65535 && D > 0 && rot >= 0 && R > 0 && P >= R + rot,
                "latent_prepare: rows %d, %d heads of %d + %d, vectors of %d in rows of %d", n, H, D, rot, R, P);
-    PL_REQUIRE(turned >= 0 && turned % 2 == 0 && turned <= rot && (turned == 0 || (cos != nullptr && sin != nullptr && table_rows > 0)),
+    PL_REQUIRE(turned >= 0 && turned % 2 == 0 && turned <= rot && (turned == 0 || (cos != nullptr && (sin == nullptr || table_rows > 0))),
                "latent_prepare: a rotation over %d of %d values", turned, rot);
     PL_REQUIRE(block_size > 0 && max_blocks > 0 && stride >= q_off + H * (D + rot) && (!write_kv || (stride >= kv_off + R + rot && gain != nullptr && pool != nullptr)),
                "latent_prepare: pages of %d, tables of %d, rows of %d values", block_size, max_blocks, stride);
@@ -216,25 +225,26 @@ extern "C" int pl_latent_prepare(const float* rows, int stride, int q_off, int k
 }
 
 // x[t, h, 0:V] *= sigmoid(g[t, h]): a gate a head on a read-out; g is 32-bit, column `g_off + h` of rows of `g_stride`.
+// `each`: a gate an element instead, x[t, e] *= sigmoid(g[t, e]).
 template <typename T>
 __global__ __launch_bounds__(256) void head_gate_kernel(T* x, const float* g, int g_stride, int g_off, const int* positions,
-                                                        int H, int V) {
+                                                        int H, int V, int each) {
     const int t = blockIdx.x;
     if (positions != nullptr && positions[t] < 0) return;
     T* row = x + static_cast<size_t>(t) * H * V;
     const float* gates = g + static_cast<size_t>(t) * g_stride + g_off;
     for (int e = threadIdx.x; e < H * V; e += 256) {
-        const float gate = 1.f / (1.f + expf(-gates[e / V]));
+        const float gate = 1.f / (1.f + expf(-gates[each ? e : e / V]));
         row[e] = from_float<T>(to_float(row[e]) * gate);
     }
 }
 
 extern "C" int pl_head_gate(void* x, int dtype, const float* g, int g_stride, int g_off, const int* positions, int n,
-                            int H, int V, hipStream_t stream) {
-    PL_REQUIRE(n >= 0 && H > 0 && V > 0 && g_off >= 0 && g_stride >= g_off + H, "head_gate: %d rows, %d heads of %d, gates at %d of %d", n, H, V, g_off, g_stride);
+                            int H, int V, int each, hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && H > 0 && V > 0 && g_off >= 0 && g_stride >= g_off + (each ? H * V : H), "head_gate: %d rows, %d heads of %d, gates at %d of %d", n, H, V, g_off, g_stride);
     if (n == 0) return 0;
-    if (dtype == PL_DTYPE_F32) head_gate_kernel<float><<<n, 256, 0, stream>>>(static_cast<float*>(x), g, g_stride, g_off, positions, H, V);
-    else if (dtype == PL_DTYPE_BF16) head_gate_kernel<bf16_t><<<n, 256, 0, stream>>>(static_cast<bf16_t*>(x), g, g_stride, g_off, positions, H, V);
+    if (dtype == PL_DTYPE_F32) head_gate_kernel<float><<<n, 256, 0, stream>>>(static_cast<float*>(x), g, g_stride, g_off, positions, H, V, each);
+    else if (dtype == PL_DTYPE_BF16) head_gate_kernel<bf16_t><<<n, 256, 0, stream>>>(static_cast<bf16_t*>(x), g, g_stride, g_off, positions, H, V, each);
     else PL_REQUIRE(false, "head_gate: dtype code %d", dtype);
     PL_CHECK_LAUNCH("head_gate");
     return 0;

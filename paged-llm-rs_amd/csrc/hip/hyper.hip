@@ -1,0 +1,277 @@
+// Several copies of the residual stream, and experts chosen by a table over token ids.
+//
+// Copies of the stream.  A model keeps S copies x_1 .. x_S of every row, [n, S, W] in 32-bit.  A sublayer
+// reads u = sum_s in[s] x_s through a norm, and its output y rebuilds every copy from all of them:
+// x_t <- sum_s mix[s, t] x_s + out[t] y.  One kernel does the rebuild behind one sublayer and the read-out
+// (with its norm) in front of the next, a row a workgroup, so that the copies travel once: either half
+// may be left out.  Sums, statistic and gain are 32-bit; the normed row is rounded once, when stored.
+//
+// Experts by table.  Row t uses the `top` experts that table[id of t] names, each weighted 1/top; an
+// expert is down(act(gate x) * (up x)).  The kernels here serve few rows, a workgroup a (row, choice):
+// a row reads only its own experts' weights.
+#include "common.hpp"
+
+#define HC_MAX_COPIES 8
+
+struct HcArgs {
+    float* streams;        // [n, S, W]
+    const float* y;        // [n, W], or null: the copies stay as they are
+    const float* mix;      // [S, S], from x to: with y
+    const float* out;      // [S]: with y
+    const float* in;       // [S], or null: nothing is read out
+    const void* gain;      // [W] 32-bit, or null: the weighted sum as it is
+    float eps;
+    void* read;            // [rows, W]: the read-out
+    const int* rows;       // which rows are read out, or null for all (with a list nothing is rebuilt)
+    int S, W;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void hc_step_kernel(HcArgs a) {
+    extern __shared__ float hc_row[];                 // the read-out's row before its norm, then 16 floats of scratch
+    float* scratch = hc_row + a.W;
+    const int i = blockIdx.x;
+    const int r = a.rows != nullptr ? a.rows[i] : i;
+    const int S = a.S, W = a.W;
+    float* x = a.streams + static_cast<size_t>(r) * S * W;
+    const float* y = a.y != nullptr ? a.y + static_cast<size_t>(r) * W : nullptr;
+    float mix[HC_MAX_COPIES * HC_MAX_COPIES], out[HC_MAX_COPIES], in[HC_MAX_COPIES];
+    if (y != nullptr) {
+#pragma unroll
+        for (int s = 0; s < HC_MAX_COPIES; ++s) {
+            out[s] = s < S ? a.out[s] : 0.f;
+#pragma unroll
+            for (int t = 0; t < HC_MAX_COPIES; ++t) mix[s * HC_MAX_COPIES + t] = (s < S && t < S) ? a.mix[s * S + t] : 0.f;
+        }
+    }
+    if (a.in != nullptr) {
+#pragma unroll
+        for (int s = 0; s < HC_MAX_COPIES; ++s) in[s] = s < S ? a.in[s] : 0.f;
+    }
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        float v[HC_MAX_COPIES];
+#pragma unroll
+        for (int s = 0; s < HC_MAX_COPIES; ++s) v[s] = s < S ? x[static_cast<size_t>(s) * W + c] : 0.f;
+        if (y != nullptr) {
+            const float add = y[c];
+            float nv[HC_MAX_COPIES];
+#pragma unroll
+            for (int t = 0; t < HC_MAX_COPIES; ++t) {
+                float acc = 0.f;
+#pragma unroll
+                for (int s = 0; s < HC_MAX_COPIES; ++s)
+                    if (s < S) acc = fmaf(mix[s * HC_MAX_COPIES + t], v[s], acc);
+                nv[t] = fmaf(out[t], add, acc);
+            }
+#pragma unroll
+            for (int t = 0; t < HC_MAX_COPIES; ++t) {
+                v[t] = nv[t];
+                if (t < S) x[static_cast<size_t>(t) * W + c] = nv[t];
+            }
+        }
+        if (a.in != nullptr) {
+            float u = 0.f;
+#pragma unroll
+            for (int s = 0; s < HC_MAX_COPIES; ++s)
+                if (s < S) u = fmaf(in[s], v[s], u);
+            hc_row[c] = u;
+            ss += u * u;
+        }
+    }
+    if (a.in == nullptr) return;
+    T* o = static_cast<T*>(a.read) + static_cast<size_t>(i) * W;
+    if (a.gain == nullptr) {
+        // (every thread reads back what it wrote itself)
+        for (int c = threadIdx.x; c < W; c += blockDim.x) o[c] = from_float<T>(hc_row[c]);
+        return;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.f / sqrtf(ss / static_cast<float>(W) + a.eps);
+    const float* gain = static_cast<const float*>(a.gain);
+    for (int c = threadIdx.x; c < W; c += blockDim.x) o[c] = from_float<T>(hc_row[c] * inv * gain[c]);
+}
+
+// streams [n, S, W] (32-bit) in place.  y, mix, out: the rebuild behind a sublayer (all null: none).  in: the
+// read-out's weights (null: none); gain (32-bit [W]) and eps: its norm (gain null: no norm); read: [rows, W] in
+// `dtype`.  rows: the rows that are read out (null: all n); with a list there is no rebuild.
+extern "C" int pl_hc_step(float* streams, const float* y, const float* mix, const float* out, const float* in,
+                          const float* gain, float eps, void* read, int dtype, const int* rows, int count, int S, int W,
+                          hipStream_t stream) {
+    PL_REQUIRE(count >= 0 && S >= 1 && S <= HC_MAX_COPIES && W > 0 && W <= 16368, "hc_step: %d rows of %d copies of %d",
+               count, S, W);
+    PL_REQUIRE((y == nullptr) == (mix == nullptr) && (y == nullptr) == (out == nullptr),
+               "hc_step: a rebuild needs the sublayer's output and both sets of weights");
+    PL_REQUIRE(rows == nullptr || y == nullptr, "hc_step: a list of rows and a rebuild");
+    PL_REQUIRE((in == nullptr) == (read == nullptr), "hc_step: a read-out needs its weights and its place");
+    if (count == 0 || (y == nullptr && in == nullptr)) return 0;
+    HcArgs a{streams, y, mix, out, in, gain, eps, read, rows, S, W};
+    const size_t lds = (static_cast<size_t>(W) + 16) * sizeof(float);
+    const int threads = W >= 1024 ? 256 : (W >= 256 ? 128 : 64);
+    if (dtype == PL_DTYPE_F32) hc_step_kernel<float><<<count, threads, lds, stream>>>(a);
+    else if (dtype == PL_DTYPE_BF16) hc_step_kernel<bf16_t><<<count, threads, lds, stream>>>(a);
+    else PL_REQUIRE(false, "hc_step: dtype code %d", dtype);
+    PL_CHECK_LAUNCH("hc_step");
+    return 0;
+}
+
+__global__ void stream_copies_kernel(const float* __restrict__ x, float* __restrict__ out, int S, int W) {
+    const size_t t = blockIdx.x;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        const float v = x[t * W + c];
+        for (int s = 0; s < S; ++s) out[(t * S + s) * W + c] = v;
+    }
+}
+
+// out[t, s, :] = x[t, :] for every s
+extern "C" int pl_stream_copies(const float* x, float* out, int n, int S, int W, hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && S >= 1 && W > 0, "stream_copies: %d rows, %d copies of %d", n, S, W);
+    if (n == 0) return 0;
+    stream_copies_kernel<<<n, 256, 0, stream>>>(x, out, S, W);
+    PL_CHECK_LAUNCH("stream_copies");
+    return 0;
+}
+
+__global__ void softcap_kernel(float* __restrict__ x, float cap, size_t count) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < count) x[i] = cap * tanhf(x[i] / cap);
+}
+
+// x = cap * tanh(x / cap)
+extern "C" int pl_softcap(float* x, float cap, long count, hipStream_t stream) {
+    PL_REQUIRE(count >= 0 && cap > 0.f, "softcap: %ld values, a cap of %g", count, static_cast<double>(cap));
+    if (count == 0) return 0;
+    softcap_kernel<<<static_cast<unsigned>((count + 255) / 256), 256, 0, stream>>>(x, cap, static_cast<size_t>(count));
+    PL_CHECK_LAUNCH("softcap");
+    return 0;
+}
+
+// ---- experts by table, few rows -------------------------------------------------------------------------
+
+// The id of row t: its own, or the one an earlier kernel left on the device (as the embedding takes it).
+__device__ __forceinline__ int moe_token(const int* ids, const int* src, const int* fed, int t) {
+    int id = ids[t];
+    if (src != nullptr) {
+        const int from = src[t];
+        if (from >= 0) id = fed[from];
+    }
+    return id;
+}
+
+// A wave's dot product of a weight row with a row of 32-bit values in LDS; every lane gets the sum.
+// The order of the additions depends on K alone.
+template <typename T>
+__device__ __forceinline__ float moe_dot(const T* __restrict__ w, const float* xs, int K, int lane) {
+    float acc = 0.f;
+    if (sizeof(T) == 2 && K % 8 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0) {
+        for (int k = lane * 8; k < K; k += 64 * 8) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(w + k);
+            const uint32_t word[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc = fmaf(__uint_as_float(word[j] << 16), xs[k + 2 * j], acc);
+                acc = fmaf(__uint_as_float(word[j] & 0xffff0000u), xs[k + 2 * j + 1], acc);
+            }
+        }
+    } else {
+        for (int k = lane; k < K; k += 64) acc = fmaf(to_float(w[k]), xs[k], acc);
+    }
+    return wave_sum(acc);
+}
+
+struct MoeArgs {
+    const void* x;         // [n, W]
+    const int* ids;
+    const int* src;
+    const int* fed;
+    const int* positions;  // rows at position -1 are padding
+    const int* table;      // [vocab, top]
+    const void* w_gu;      // [E, 2 F, W]: an expert's gate rows, then its up rows
+    const void* w_down;    // [E, W, F]
+    void* h;               // [n, top, F]
+    float* out;            // [n, W]
+    int n, W, F, E, top, vocab, act;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_up_kernel(MoeArgs a) {
+    extern __shared__ float moe_x[];
+    const int t = blockIdx.x / a.top, c = blockIdx.x % a.top;
+    if (a.positions[t] < 0) return;
+    const int id = moe_token(a.ids, a.src, a.fed, t);
+    if (id < 0 || id >= a.vocab) return;
+    const int e = a.table[static_cast<size_t>(id) * a.top + c];
+    if (e < 0 || e >= a.E) return;
+    const int W = a.W, F = a.F;
+    const T* x = static_cast<const T*>(a.x) + static_cast<size_t>(t) * W;
+    for (int k = threadIdx.x; k < W; k += blockDim.x) moe_x[k] = to_float(x[k]);
+    __syncthreads();
+    const int lane = threadIdx.x % PL_WAVE, wave = threadIdx.x / PL_WAVE, waves = blockDim.x / PL_WAVE;
+    const T* gate = static_cast<const T*>(a.w_gu) + static_cast<size_t>(e) * 2 * F * W;
+    const T* up = gate + static_cast<size_t>(F) * W;
+    T* h = static_cast<T*>(a.h) + (static_cast<size_t>(t) * a.top + c) * F;
+    for (int f = blockIdx.y * waves + wave; f < F; f += gridDim.y * waves) {
+        const float g = moe_dot<T>(gate + static_cast<size_t>(f) * W, moe_x, W, lane);
+        const float u = moe_dot<T>(up + static_cast<size_t>(f) * W, moe_x, W, lane);
+        if (lane == 0) h[f] = from_float<T>(pl_activate<true>(g, a.act) * u);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_kernel(MoeArgs a) {
+    extern __shared__ float moe_h[];                  // [top, F]
+    const int t = blockIdx.x;
+    const int W = a.W, F = a.F, top = a.top;
+    float* o = a.out + static_cast<size_t>(t) * W;
+    const int lane = threadIdx.x % PL_WAVE, wave = threadIdx.x / PL_WAVE, waves = blockDim.x / PL_WAVE;
+    const int id = a.positions[t] < 0 ? -1 : moe_token(a.ids, a.src, a.fed, t);
+    if (id < 0 || id >= a.vocab) {
+        for (int w = blockIdx.y * blockDim.x + threadIdx.x; w < W; w += gridDim.y * blockDim.x) o[w] = 0.f;
+        return;
+    }
+    const T* h = static_cast<const T*>(a.h) + static_cast<size_t>(t) * top * F;
+    for (int k = threadIdx.x; k < top * F; k += blockDim.x) moe_h[k] = to_float(h[k]);
+    __syncthreads();
+    const float share = 1.f / static_cast<float>(top);
+    for (int w = blockIdx.y * waves + wave; w < W; w += gridDim.y * waves) {
+        float sum = 0.f;
+        for (int c = 0; c < top; ++c) {
+            const int e = a.table[static_cast<size_t>(id) * top + c];
+            if (e < 0 || e >= a.E) continue;
+            const T* down = static_cast<const T*>(a.w_down) + (static_cast<size_t>(e) * W + w) * F;
+            sum += moe_dot<T>(down, moe_h + c * F, F, lane) * share;
+        }
+        if (lane == 0) o[w] = sum;
+    }
+}
+
+// out[t] (32-bit) = (1/top) sum over the experts e that table[id of t] names of down_e (act(gate_e x_t) * (up_e x_t)).
+// x [n, W], w_gu [E, 2 F, W], w_down [E, W, F] and the workspace h [n, top, F] in `dtype`; table [vocab, top].
+extern "C" int pl_moe_rows(const void* x, const int* ids, const int* src, const int* fed, const int* positions,
+                           const int* table, const void* w_gu, const void* w_down, void* h, float* out, int dtype,
+                           int n, int W, int F, int E, int top, int vocab, int act, hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && W > 0 && F > 0 && E > 0 && top > 0 && top <= E && vocab > 0 && act >= 0 && act <= 2,
+               "moe_rows: %d rows of %d, %d experts of %d, %d a row", n, W, E, F, top);
+    PL_REQUIRE((src == nullptr) == (fed == nullptr), "moe_rows: rows fed from the step before need both the rows and the tokens");
+    PL_REQUIRE(W <= 16384 && static_cast<long long>(top) * F <= 16384, "moe_rows: rows of %d, %d experts of %d a row", W, top, F);
+    PL_REQUIRE(static_cast<long long>(n) * top < (1ll << 31), "moe_rows: %d rows", n);
+    if (n == 0) return 0;
+    MoeArgs a{x, ids, src, fed, positions, table, w_gu, w_down, h, out, n, W, F, E, top, vocab, act};
+    // few rows: deal an expert's rows of weights to several workgroups, so that the chip has work
+    const int cu = pl_compute_units();
+    int up_parts = 1, down_parts = 1;
+    while (static_cast<long long>(n) * top * up_parts < 2ll * cu && up_parts * 8 < F) up_parts *= 2;
+    while (static_cast<long long>(n) * down_parts < 2ll * cu && down_parts * 8 < W) down_parts *= 2;
+    const dim3 up_grid(n * top, up_parts), down_grid(n, down_parts);
+    if (dtype == PL_DTYPE_F32) {
+        moe_up_kernel<float><<<up_grid, 256, W * sizeof(float), stream>>>(a);
+        moe_down_kernel<float><<<down_grid, 256, static_cast<size_t>(top) * F * sizeof(float), stream>>>(a);
+    } else if (dtype == PL_DTYPE_BF16) {
+        moe_up_kernel<bf16_t><<<up_grid, 256, W * sizeof(float), stream>>>(a);
+        moe_down_kernel<bf16_t><<<down_grid, 256, static_cast<size_t>(top) * F * sizeof(float), stream>>>(a);
+    } else {
+        PL_REQUIRE(false, "moe_rows: dtype code %d", dtype);
+    }
+    PL_CHECK_LAUNCH("moe_rows");
+    return 0;
+}

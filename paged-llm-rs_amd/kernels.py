@@ -39,7 +39,7 @@ def _signatures(lib) -> None:
         "pl_gemm_heads": [p, p, p, i, i, i, i, i, ctypes.c_long, i, ctypes.c_long, i, i, p],
         "pl_head_prepare": [p, i, i, i, f, p, p, p, p, i, i, i, i, f, i, p, p, p, i, i, i, p, p, p, i, i, i, i, i, i, i, p],
         "pl_latent_prepare": [p, i, i, i, p, f, p, p, i, i, p, p, p, i, i, i, p, p, p, i, i, i, i, i, i, i, p],
-        "pl_head_gate": [p, i, p, i, i, p, i, i, i, p],
+        "pl_head_gate": [p, i, p, i, i, p, i, i, i, i, p],
         "pl_add_position_rows": [p, p, i, p, i, i, i, p],
         "pl_paged_attention_prefill_tile": [i, i],
         "pl_argmax": [p, p, p, p, i, i, p],
@@ -75,6 +75,10 @@ def _signatures(lib) -> None:
         "pl_to_bf16": [p, p, ctypes.c_long, p],
         "pl_activation": [p, p, i, i, ctypes.c_long, p],
         "pl_weighted_sum": [p, f, p, f, ctypes.c_long, p],
+        "pl_hc_step": [p, p, p, p, p, p, f, p, i, p, i, i, i, p],
+        "pl_stream_copies": [p, p, i, i, i, p],
+        "pl_softcap": [p, f, ctypes.c_long, p],
+        "pl_moe_rows": [p, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, p],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name)
@@ -1414,7 +1418,10 @@ def latent_prepare(rows: torch.Tensor, q_off: int, kv_off: int, gain, eps: float
     if write_kv:
         _need(gain, "gain of the small vector", (R,), torch.float32)
     table_rows = 0
-    if turned:
+    if turned and sin is None:
+        # no tables: ``cos`` lists the frequencies and the kernel works the angles out (position * frequency in 32-bit)
+        _need(cos, "rotation frequencies", (turned // 2,), torch.float32)
+    elif turned:
         _need(cos, "cosine table", None, torch.float32)
         _need(sin, "sine table", tuple(cos.shape), torch.float32)
         if cos.dim() != 2 or cos.shape[1] != turned // 2:
@@ -1428,15 +1435,18 @@ def latent_prepare(rows: torch.Tensor, q_off: int, kv_off: int, gain, eps: float
         n, H, D, rot, R, padded, _stream()))
 
 
-def head_gate_(x: torch.Tensor, rows: torch.Tensor, off: int, positions, H: int, V: int) -> torch.Tensor:
-    """x[t, h, :] *= sigmoid(rows[t, off + h]) in place; ``x`` [n, H * V], ``rows`` 32-bit."""
+def head_gate_(x: torch.Tensor, rows: torch.Tensor, off: int, positions, H: int, V: int,
+               each_element: bool = False) -> torch.Tensor:
+    """x[t, h, :] *= sigmoid(rows[t, off + h]) in place; ``x`` [n, H * V], ``rows`` 32-bit.  ``each_element``:
+    a gate an element instead of a head, x[t, e] *= sigmoid(rows[t, off + e])."""
     n = x.shape[0]
+    gates = H * V if each_element else H
     _need(x, "read-outs", (n, H * V))
     _need(rows, "gate rows", None, torch.float32)
-    if rows.dim() != 2 or rows.shape[0] != n or rows.shape[1] < off + H:
-        raise TensorError(f"gate rows of shape {tuple(rows.shape)} for {n} tokens and {H} gates from column {off}")
+    if rows.dim() != 2 or rows.shape[0] != n or rows.shape[1] < off + gates:
+        raise TensorError(f"gate rows of shape {tuple(rows.shape)} for {n} tokens and {gates} gates from column {off}")
     _check(library().pl_head_gate(x.data_ptr(), _code(x, "read-outs"), rows.data_ptr(), rows.shape[1], int(off),
-                                  _ptr(positions), n, H, V, _stream()))
+                                  _ptr(positions), n, H, V, 1 if each_element else 0, _stream()))
     return x
 
 
@@ -1459,3 +1469,84 @@ def sink_attention(q: torch.Tensor, out: torch.Tensor, batch, kv, nq: int, nkv: 
     head on the distance; ``q`` [n, nq * d] holds the prepared queries.  In bfloat16 the matrix-core kernel for
     portions and the kernels for single tokens, for head sizes they take; the plain kernel otherwise."""
     return paged_attention(q, out, batch, kv, nq, nkv, d, scale, window, sinks=sinks, slopes=slopes)
+
+
+# ---- several copies of the stream; experts chosen by a table over token ids ------------------------------------
+
+HC_MAX_COPIES = 8
+
+
+def stream_copies(x: torch.Tensor, copies: int) -> torch.Tensor:
+    """[n, copies * W]: every row of the 32-bit stream ``x`` [n, W] ``copies`` times, one behind the other."""
+    n, W = x.shape
+    _need(x, "stream", None, torch.float32)
+    out = torch.empty((n, copies * W), dtype=torch.float32, device=x.device)
+    _check(library().pl_stream_copies(x.data_ptr(), out.data_ptr(), n, int(copies), W, _stream()))
+    return out
+
+
+def hc_step(streams: torch.Tensor, copies: int, y=None, mix=None, out=None, read=None, gain=None, eps: float = 0.0,
+            read_dtype: torch.dtype = torch.float32, rows=None):
+    """One pass over the copies of the stream, ``streams`` [n, copies * W] in 32-bit, with either half optional.
+    Rebuild (``y`` [n, W] 32-bit, ``mix`` [copies, copies], ``out`` [copies]): copy t becomes
+    sum_s mix[s, t] x_s + out[t] y, in place.  Read-out (``read`` [copies]): u = sum_s read[s] x_s of the rebuilt
+    copies, normed with ``gain`` (32-bit [W]) and ``eps`` where a gain is given, comes back as [rows, W] in
+    ``read_dtype`` (None where nothing is read out).  ``rows``: the rows to read out (then nothing is rebuilt)."""
+    n = streams.shape[0]
+    _need(streams, "copies of the stream", None, torch.float32)
+    if streams.dim() != 2 or streams.shape[1] % copies or not 1 <= copies <= HC_MAX_COPIES:
+        raise TensorError(f"{copies} copies of the stream in rows of {tuple(streams.shape)}")
+    W = streams.shape[1] // copies
+    if y is not None:
+        _need(y, "sublayer output", (n, W), torch.float32)
+        _need(mix, "weights between the copies", (copies, copies), torch.float32)
+        _need(out, "weights of the sublayer output", (copies,), torch.float32)
+        if rows is not None:
+            raise TensorError("a list of rows and a rebuild of the copies")
+    result = None
+    count = n
+    if read is not None:
+        _need(read, "weights of the read-out", (copies,), torch.float32)
+        if gain is not None:
+            _need(gain, "gain of the read-out's norm", (W,), torch.float32)
+        if rows is not None:
+            _need(rows, "rows to read out", None, torch.int32)
+            count = rows.numel()
+        result = torch.empty((count, W), dtype=read_dtype, device=streams.device)
+    elif y is None:
+        return None
+    _check(library().pl_hc_step(streams.data_ptr(), _ptr(y), _ptr(mix), _ptr(out), _ptr(read), _ptr(gain), float(eps),
+                                _ptr(result), _CODES[read_dtype], _ptr(rows), count, int(copies), W, _stream()))
+    return result
+
+
+def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x <- cap * tanh(x / cap) on 32-bit values, in place."""
+    _need(x, "logits", None, torch.float32)
+    _check(library().pl_softcap(x.data_ptr(), float(cap), x.numel(), _stream()))
+    return x
+
+
+def moe_rows(x: torch.Tensor, batch, table: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
+             activation: str = "silu") -> torch.Tensor:
+    """Experts chosen by a table over token ids, a row at a time: 32-bit [n, W], row t the mean over the experts e
+    that ``table[id of t]`` names of down_e (act(gate_e x_t) * (up_e x_t)).  ``w_gate_up`` [E, 2 F, W] (an expert's
+    gate rows, then its up rows), ``w_down`` [E, W, F], of ``x``'s type; ``table`` [vocabulary, top] int32.  A row's
+    id is the batch's, or the one an earlier step left on the device; padding rows give zeros."""
+    n, W = x.shape
+    _need(x, "rows")
+    E, F2, _ = w_gate_up.shape
+    F = F2 // 2
+    _need(w_gate_up, "gate and up weights of the experts", (E, 2 * F, W), x.dtype)
+    _need(w_down, "down weights of the experts", (E, W, F), x.dtype)
+    _need(table, "table of experts", None, torch.int32)
+    vocab, top = table.shape
+    fed = getattr(batch, "fed_tokens", None)
+    src = batch.token_src if fed is not None else None
+    h = torch.empty((n, top, F), dtype=x.dtype, device=x.device)
+    out = torch.empty((n, W), dtype=torch.float32, device=x.device)
+    _check(library().pl_moe_rows(x.data_ptr(), batch.token_ids.data_ptr(), _ptr(src), _ptr(fed),
+                                 batch.positions.data_ptr(), table.data_ptr(), w_gate_up.data_ptr(), w_down.data_ptr(),
+                                 h.data_ptr(), out.data_ptr(), _code(x, "rows"), n, W, F, E, top, vocab,
+                                 activation_code(activation), _stream()))
+    return out

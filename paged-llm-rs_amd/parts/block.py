@@ -293,3 +293,111 @@ class SharedNormBlock:
 
 
 register_block("shared_norm", SharedNormBlock)
+
+
+class HyperConnectionBlock:
+    """The pre-norm arrangement over several copies of the stream.  The stream a layer gets is [rows, S * width]:
+    S copies x_1 .. x_S of every row, one behind the other.  A sublayer (1: the mixer, 2: the feed-forward, where
+    the layer has one) reads u = sum_s in[s] x_s through its norm, and its output y rebuilds every copy from all
+    of them, x_t <- sum_s mix[s, t] x_s + out[t] y.  A layer spec without ``stream_copies`` has the one stream
+    and the plain sums x <- x + y, computed as one copy with weights of one.
+
+    Everything about the copies is 32-bit.  One kernel rebuilds the copies behind a sublayer and reads out the
+    next sublayer's normed rows in the same pass (``kernels.hc_step``).  Sublayers hand back 32-bit rows.
+    Tensor names: the norms' gains under the norms' own names; ``hc1.in`` [S], ``hc1.out`` [S], ``hc1.mix`` [S, S]
+    (from, to) for the mixer and ``hc2.*`` for the feed-forward."""
+
+    NAMES = {"norm1": "norm1", "mixer": "mix", "norm2": "norm2", "feed_forward": "mlp", "copies1": "hc1", "copies2": "hc2"}
+
+    @classmethod
+    def names_of(cls, layer) -> dict:
+        given = getattr(layer, "names", None) or {}
+        unknown = sorted(set(given) - set(cls.NAMES))
+        if unknown:
+            raise ConfigError(f"a layer names members that this arrangement does not have: {unknown}")
+        return {**cls.NAMES, **given}
+
+    @staticmethod
+    def _copy_decls(name: str, copies: int) -> list:
+        from ..weights.loader import ParamDecl
+
+        return [ParamDecl(f"{name}.in", (copies,), "copy_in"), ParamDecl(f"{name}.out", (copies,), "copy_out"),
+                ParamDecl(f"{name}.mix", (copies, copies), "copy_mix")]
+
+    @classmethod
+    def declare(cls, layer, hidden: int) -> list:
+        from ..weights.loader import ParamDecl
+
+        n = cls.names_of(layer)
+        copies = layer.stream_copies
+        mixer = lookup(MIXERS, layer.mixer.kind, "mixer")
+        gain = lookup(NORMS, layer.norm.kind, "norm").declare(layer.norm, hidden)[0].role
+        decls = [ParamDecl(n["norm1"], (hidden,), gain)] + prefixed(mixer.declare(layer.mixer, hidden), n["mixer"])
+        if copies is not None:
+            decls += cls._copy_decls(n["copies1"], copies)
+        if layer.feed_forward is not None:
+            ffn = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")
+            decls += [ParamDecl(n["norm2"], (hidden,), gain)] + prefixed(ffn.declare(layer.feed_forward, hidden), n["feed_forward"])
+            if copies is not None:
+                decls += cls._copy_decls(n["copies2"], copies)
+        return decls
+
+    def __init__(self, layer, hidden: int, params: dict, dtype, device, shared: dict):
+        n = self.names = self.names_of(layer)
+        norm = lookup(NORMS, layer.norm.kind, "norm")
+        if not getattr(norm, "fuses_into_product", False):
+            raise ConfigError(f"norm {layer.norm.kind!r} cannot run inside the pass over the copies of the stream "
+                              "(it needs a 32-bit gain and an eps, nothing else)")
+        self.dtype, self.hidden = dtype, hidden
+        self.copies = int(layer.stream_copies or 1)
+        if not 1 <= self.copies <= kernels.HC_MAX_COPIES:
+            raise ConfigError(f"{self.copies} copies of the stream (1 to {kernels.HC_MAX_COPIES})")
+        self.norm1 = norm(layer.norm, hidden, {"weight": params[n["norm1"]]}, dtype, device)
+        self.mixer = lookup(MIXERS, layer.mixer.kind, "mixer")(
+            layer.mixer, hidden, scoped(params, n["mixer"]), dtype, device, shared)
+        self.weights1 = self._copy_weights(params, n["copies1"], layer.stream_copies, device)
+        self.norm2 = self.feed_forward = self.weights2 = None
+        if layer.feed_forward is not None:
+            self.norm2 = norm(layer.norm, hidden, {"weight": params[n["norm2"]]}, dtype, device)
+            self.feed_forward = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")(
+                layer.feed_forward, hidden, scoped(params, n["feed_forward"]), dtype, device, shared)
+            self.weights2 = self._copy_weights(params, n["copies2"], layer.stream_copies, device)
+
+    @staticmethod
+    def _copy_weights(params: dict, name: str, copies, device) -> tuple:
+        """(in, mix, out) in 32-bit; for the one plain stream all three are one."""
+        if copies is None:
+            one = torch.ones((1,), dtype=torch.float32, device=device)
+            return one, one.view(1, 1), one
+        return tuple(params[f"{name}.{part}"].to(torch.float32).contiguous() for part in ("in", "mix", "out"))
+
+    @property
+    def graph_safe(self) -> bool:
+        return getattr(self.mixer, "graph_safe", True) and getattr(self.feed_forward, "graph_safe", True)
+
+    def _feed(self, rows, ctx):
+        ffn = self.feed_forward
+        if getattr(ffn, "takes_batch", False):
+            return ffn.forward(rows, batch=ctx.batch)
+        return ffn.forward(rows)
+
+    def forward(self, resid, delta, ctx):
+        if delta is not None:
+            raise ConfigError("a layer over copies of the stream behind a layer that left its output unadded")
+        if resid.shape[1] != self.copies * self.hidden:
+            raise ConfigError(f"a stream of rows of {resid.shape[1]} for {self.copies} copies of {self.hidden}")
+        S = self.copies
+        in1, mix1, out1 = self.weights1
+        rows = kernels.hc_step(resid, S, read=in1, gain=self.norm1.gain32, eps=self.norm1.eps, read_dtype=self.dtype)
+        mixed = self.mixer.forward(rows, ctx)
+        if self.feed_forward is None:
+            kernels.hc_step(resid, S, y=mixed, mix=mix1, out=out1)
+            return None
+        in2, mix2, out2 = self.weights2
+        rows = kernels.hc_step(resid, S, y=mixed, mix=mix1, out=out1, read=in2, gain=self.norm2.gain32,
+                               eps=self.norm2.eps, read_dtype=self.dtype)
+        kernels.hc_step(resid, S, y=self._feed(rows, ctx), mix=mix2, out=out2)
+        return None
+
+
+register_block("hyper_connections", HyperConnectionBlock)

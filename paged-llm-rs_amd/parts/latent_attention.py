@@ -47,7 +47,7 @@ class LatentAttention:
         if spec.sink == "learned":
             decls.append(ParamDecl("sink", (H,), "bias"))
         if spec.gated:
-            decls.append(ParamDecl("g", (H, hidden)))
+            decls.append(ParamDecl("g", (H * V if spec.gate_each == "element" else H, hidden)))
         decls.append(ParamDecl("o", (hidden, H * V)))
         return decls
 
@@ -59,6 +59,8 @@ class LatentAttention:
             raise UnsupportedError(f"vectors of {R} with a rotated part of {rot}: the attention kernels take rows up to 1024")
         if spec.rotary_turned % 2 or not 0 <= spec.rotary_turned <= rot:
             raise UnsupportedError(f"a rotation over {spec.rotary_turned} values of a part of {rot}")
+        if spec.gate_each not in ("head", "element"):
+            raise UnsupportedError(f"a gate a {spec.gate_each!r} (head or element)")
         self.spec, self.dtype = spec, dtype
         self.H, self.D, self.rot, self.V, self.R = H, D, rot, V, R
         self.scale = float(spec.scale) if spec.scale is not None else 1.0 / math.sqrt(D + rot)
@@ -80,10 +82,17 @@ class LatentAttention:
         self.uk_t = params["uk"].view(H, D, R).transpose(1, 2).contiguous()
         self.uv = params["uv"].view(H, V, R).contiguous()
         self.sinks = head_sinks(spec.sink, H, params, device)
-        self.rotary = None
-        if spec.rotary_turned:
-            self.rotary = rotary_tables(PositionSpec("rotary_neighbours", spec.rotary_turned, float(spec.rotary_base),
-                                                     int(spec.max_positions)), device, shared)
+        # the rotation's angles: tables of cosines and sines where the spec bounds the positions, otherwise the
+        # frequencies alone (rounded from 64-bit), and the kernel multiplies by the position in 32-bit
+        self.cos = self.sin = None
+        if spec.rotary_turned and spec.max_positions:
+            rotary = rotary_tables(PositionSpec("rotary_neighbours", spec.rotary_turned, float(spec.rotary_base),
+                                                int(spec.max_positions)), device, shared)
+            self.cos, self.sin = rotary.cos, rotary.sin
+        elif spec.rotary_turned:
+            turned = spec.rotary_turned
+            self.cos = torch.tensor([float(spec.rotary_base) ** (-2.0 * i / turned) for i in range(turned // 2)],
+                                    dtype=torch.float64).to(torch.float32).to(device)
         self.o_proj = Linear(params["o"])
 
     def cache_spec(self):
@@ -101,9 +110,7 @@ class LatentAttention:
         n = rows.shape[0]
         q = torch.empty((n, H * P), dtype=self.dtype, device=rows.device)
         q_plain = torch.empty((H, n, D), dtype=self.dtype, device=rows.device)
-        cos = self.rotary.cos if self.rotary is not None else None
-        sin = self.rotary.sin if self.rotary is not None else None
-        kernels.latent_prepare(rows, 0, self.kv_off, self.gain, self.spec.norm_eps, cos, sin, self.spec.rotary_turned,
+        kernels.latent_prepare(rows, 0, self.kv_off, self.gain, self.spec.norm_eps, self.cos, self.sin, self.spec.rotary_turned,
                                batch, kv, q_plain, q, H, D, rot, R, P,
                                write_kv=ctx.writes_cache and not self.spec.borrows)
         kernels.gemm_heads(q_plain.transpose(0, 1), self.uk_t, q.view(n, H, P)[:, :, :R])
@@ -112,7 +119,8 @@ class LatentAttention:
         values = torch.empty((n, H * V), dtype=self.dtype, device=rows.device)
         kernels.gemm_heads(out.view(n, H, P)[:, :, :R], self.uv, values.view(n, H, V))
         if self.spec.gated:
-            kernels.head_gate_(values, rows, self.gate_off, batch.positions, H, V)
+            kernels.head_gate_(values, rows, self.gate_off, batch.positions, H, V,
+                               each_element=self.spec.gate_each == "element")
         return self.o_proj.forward(values, out_dtype=torch.float32, add_into=getattr(ctx, "residual", None))
 
 

@@ -97,3 +97,48 @@ class DenseMlp:
 
 
 register_feed_forward("dense_mlp", DenseMlp)
+
+
+class TableExperts:
+    """Small gated feed-forwards of which a token uses the few that a table names for its id, each with the
+    same weight: the mean over the chosen e of down_e(act(gate_e x) * (up_e x)).  Nothing is learned about the
+    choice and nothing depends on the other rows of the step.  The result comes back in 32-bit.
+    Tensors: ``e<i>.gate``, ``e<i>.up`` [ff, width], ``e<i>.down`` [width, ff]; ``table`` [vocabulary, top], integers."""
+
+    # forward needs the step's token ids
+    takes_batch = True
+    graph_safe = True
+
+    @staticmethod
+    def declare(spec, hidden: int) -> list:
+        decls = []
+        for e in range(spec.experts):
+            decls += [ParamDecl(f"e{e}.gate", (spec.intermediate_size, hidden)),
+                      ParamDecl(f"e{e}.up", (spec.intermediate_size, hidden)),
+                      ParamDecl(f"e{e}.down", (hidden, spec.intermediate_size))]
+        decls.append(ParamDecl("table", (spec.vocab_size, spec.top), f"choice_table:{spec.experts}"))
+        return decls
+
+    def __init__(self, spec, hidden: int, params: dict, dtype, device, shared: dict):
+        if spec.activation not in kernels.ACTIVATIONS:
+            raise UnsupportedError(f"activation {spec.activation!r}, the kernels know {', '.join(sorted(kernels.ACTIVATIONS))}")
+        if not 1 <= spec.top <= spec.experts:
+            raise UnsupportedError(f"{spec.top} of {spec.experts} experts a token")
+        self.spec, self.activation = spec, spec.activation
+        E = spec.experts
+        # [E, 2 F, W]: an expert's gate rows, then its up rows; [E, W, F]
+        self.w_gate_up = torch.stack([torch.cat([params[f"e{e}.gate"], params[f"e{e}.up"]], 0) for e in range(E)]).contiguous()
+        self.w_down = torch.stack([params[f"e{e}.down"] for e in range(E)]).contiguous()
+        table = params["table"]
+        if table.dtype != torch.int32:
+            raise UnsupportedError(f"a table of experts of type {table.dtype}")
+        low, high = int(table.min()), int(table.max())
+        if low < 0 or high >= E:
+            raise UnsupportedError(f"the table of experts names experts {low} to {high} of {E}")
+        self.table = table.contiguous()
+
+    def forward(self, x, batch):
+        return kernels.moe_rows(x, batch, self.table, self.w_gate_up, self.w_down, self.activation)
+
+
+register_feed_forward("table_experts", TableExperts)

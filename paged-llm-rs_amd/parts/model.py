@@ -19,7 +19,7 @@ from ..weights.loader import ParamDecl, load_weights
 from . import attention, block, conv_attention, latent_attention, mlp, norm, parallel, recurrent, sink_attention, transforms  # noqa: F401  (register the built-in parts)
 from .linear import Linear, linears_of
 from .norm import PendingNorm
-from .registry import BLOCKS, EMBED_TRANSFORMS, LOGIT_TRANSFORMS, NORMS, lookup, prefixed, scoped
+from .registry import BLOCKS, EMBED_TRANSFORMS, FINAL_TRANSFORMS, LOGIT_TRANSFORMS, NORMS, lookup, prefixed, scoped
 from .trace import ActivationTrace
 
 DTYPES = {"float32": torch.float32, "f32": torch.float32, "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
@@ -40,10 +40,11 @@ class TransformChain:
 
 
 def _transforms(spec) -> list:
-    """(attribute, classes) of the transforms the spec names: of the stream behind the embedding and of the
-    logits.  A spec names one transform or a list of them, applied in that order."""
+    """(attribute, classes) of the transforms the spec names: of the stream behind the embedding, of the stream
+    before the final norm and of the logits.  A spec names one transform or a list of them, applied in that order."""
     found = []
     for key, registry, what in (("embed_transform", EMBED_TRANSFORMS, "embedding transform"),
+                                ("final_transform", FINAL_TRANSFORMS, "transform before the final norm"),
                                 ("logit_transform", LOGIT_TRANSFORMS, "logit transform")):
         kind = (spec.extra or {}).get(key)
         if kind is not None:
@@ -94,6 +95,9 @@ class LayerContext:
                  "norm_after", "handed_out", "stream_rows")
 
     def __init__(self, batch, cache, layer: int, cache_layer: int, writes_cache: bool):
+        # ``layer`` and ``cache_layer`` are the keys under which the cache keeps this run's state and the pages it
+        # reads: a layer's index, or, for a layer that runs several times with pages and state for every run, the
+        # key the schedule gives that run
         self.batch = batch
         self.cache = cache
         self.layer = layer
@@ -149,18 +153,19 @@ class DecoderModel:
         else:
             raise WeightError(f"no {spec.head_name}, and the config does not tie the embeddings")
         self.lm_head = Linear(head)
-        self.embed_transform = self.logit_transform = None
+        self.embed_transform = self.final_transform = self.logit_transform = None
         for key, classes in _transforms(spec):
             members = [cls(spec, params, dtype, self.device) for cls in classes]
             setattr(self, key, members[0] if len(members) == 1 else TransformChain(members))
         for entry in spec.schedule:
             if not 0 <= entry.layer < len(self.blocks):
                 raise ConfigError(f"the schedule names layer {entry.layer} of {len(self.blocks)}")
-            if entry.cache_from is not None and not 0 <= entry.cache_from < len(self.blocks):
-                raise ConfigError(f"the schedule reads the cache of layer {entry.cache_from} of {len(self.blocks)}")
+            if entry.cache_from is not None and entry.cache_key is not None:
+                raise ConfigError(f"a run of layer {entry.layer} both keeps a cache of its own and reads another's")
         self.cache_layout = CacheLayout.from_blocks(self.blocks, spec.schedule)
         self.graph_safe = (all(getattr(b, "graph_safe", True) for b in self.blocks)
                            and getattr(self.embed_transform, "graph_safe", True)
+                           and getattr(self.final_transform, "graph_safe", True)
                            and getattr(self.logit_transform, "graph_safe", True))
         # Mixers that hand requests of few tokens to a kernel of their own say from how many tokens on a
         # request counts as a long portion; a step reports the tokens of the shorter ones for each such limit.
@@ -211,7 +216,8 @@ class DecoderModel:
         schedule = self.spec.schedule
         for at, entry in enumerate(schedule):
             own = entry.cache_from is None
-            ctx = LayerContext(batch, cache, entry.layer, entry.layer if own else entry.cache_from, own)
+            key = entry.layer if entry.cache_key is None else entry.cache_key
+            ctx = LayerContext(batch, cache, key, key if own else entry.cache_from, own)
             if top is not None:
                 ctx.trace = top.child(self.spec.layers[entry.layer].weight_prefix)
             ctx.handed = handed
@@ -231,10 +237,16 @@ class DecoderModel:
             # A portion in the middle of a prompt runs only to fill the cache.
             # Nothing further is launched for it.
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+        rows = batch.logit_rows
+        if self.final_transform is not None:
+            if delta is not None:
+                kernels.residual_add(resid, delta)
+                delta = None
+            resid, rows = self.final_transform(resid, batch), None      # [wanted rows, hidden]
         if delta is None:
-            normed = PendingNorm(self.norm, resid, self.dtype, rows=batch.logit_rows)
+            normed = PendingNorm(self.norm, resid, self.dtype, rows=rows)
         else:
-            normed = self.norm.apply(resid, delta, self.dtype, rows=batch.logit_rows)
+            normed = self.norm.apply(resid, delta, self.dtype, rows=rows)
         if top is not None:
             if isinstance(normed, PendingNorm):
                 normed = normed.materialize()

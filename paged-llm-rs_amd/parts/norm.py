@@ -37,19 +37,24 @@ class PendingNorm:
 
 
 class RmsNorm:
-    """x / sqrt(mean(x^2) + eps) * gain, statistic and product in 32-bit."""
+    """x / sqrt(mean(x^2) + eps) * gain, statistic and product in 32-bit.  A spec with a ``gain_offset`` stores
+    its gains as distances from that number (gains around zero for an offset of one): the sum is taken once,
+    in 32-bit, when the norm is built."""
 
     # a product kernel can take this norm as its first stage: it needs ``gain32`` and ``eps`` only
     fuses_into_product = True
 
     @staticmethod
     def declare(spec, width: int) -> list:
-        return [ParamDecl("weight", (width,), "gain")]
+        return [ParamDecl("weight", (width,), "gain_around_zero" if getattr(spec, "gain_offset", 0.0) else "gain")]
 
     def __init__(self, spec, width: int, params: dict, dtype, device):
         self.eps = float(spec.eps)
         self.width = width
         self.gain = params["weight"]
+        offset = float(getattr(spec, "gain_offset", 0.0) or 0.0)
+        if offset:
+            self.gain = (self.gain.to(torch.float32) + offset).contiguous()
         # the product kernels that take the norm as their first stage read the gain in 32-bit
         self.gain32 = self.gain if self.gain.dtype == torch.float32 else self.gain.float()
 

@@ -28,6 +28,10 @@ transform     of the stream behind the embedding (``register_embed_transform``) 
               ``__init__(spec, params, dtype, device)`` (``params``: all tensors by checkpoint name);
               ``__call__(x, batch) -> x``: the 32-bit stream [rows, hidden] (padding rows have
               position -1), or the 32-bit logits [wanted rows, vocabulary]; it may work in place.
+              A third kind (``register_final_transform``, ``extra["final_transform"]``) stands between the
+              last layer and the final norm: it gets the stream as the layers leave it and gives the rows
+              whose logits are wanted, [wanted rows, hidden] in 32-bit (the sum of several copies of the
+              stream, say); the final norm then reads every row of what it gives.
 """
 
 from __future__ import annotations
@@ -41,6 +45,7 @@ BLOCKS: dict = {}
 POSITIONS: dict = {}
 EMBED_TRANSFORMS: dict = {}
 LOGIT_TRANSFORMS: dict = {}
+FINAL_TRANSFORMS: dict = {}
 
 
 def register_mixer(kind: str, cls) -> None:
@@ -69,6 +74,10 @@ def register_embed_transform(kind: str, cls) -> None:
 
 def register_logit_transform(kind: str, cls) -> None:
     LOGIT_TRANSFORMS[kind] = cls
+
+
+def register_final_transform(kind: str, cls) -> None:
+    FINAL_TRANSFORMS[kind] = cls
 
 
 def lookup(registry: dict, kind: str, what: str):

@@ -1,7 +1,8 @@
-"""Grouped-query softmax attention over the paged cache with a sink in the softmax's denominator and,
-as the spec asks, q and k as unit vectors (divided by their root mean square over a head, no gain), a
-query temperature that grows with the logarithm of the position, a penalty a head on the distance
-between query and key, and a window.
+"""Grouped-query softmax attention over the paged cache with, as the spec asks, a sink in the softmax's
+denominator, q and k as unit vectors (divided by their root mean square over a head, with or without a
+gain), biases on the projections, a query temperature that grows with the logarithm of the position, a
+penalty a head on the distance between query and key, and a window or a mask of blocks (a query sees the
+keys of its own block of positions, blocks counted from the request's position 0).
 
 weights_ij = exp(s_ij) / (exp(sink_h) + sum over the visible j of exp(s_ij)),
 s_ij = scale (q_i . k_j) - slope_h (i - j); a sink has no key and no value, so a row's weights sum to
@@ -60,10 +61,18 @@ class SinkAttention:
                  ParamDecl("o", (hidden, H * V))]
         if spec.sink == "learned":
             decls.append(ParamDecl("sink", (H,), "bias"))
+        if spec.qk_gain:
+            decls += [ParamDecl("q.norm", (D,), "gain"), ParamDecl("k.norm", (D,), "gain")]
+        if spec.qkv_bias:
+            decls += [ParamDecl("q.b", (H * D,), "bias"), ParamDecl("k.b", (G * D,), "bias"), ParamDecl("v.b", (G * V,), "bias")]
         return decls
 
     def __init__(self, spec, hidden: int, params: dict, dtype, device, shared: dict):
         H, G, D, V = spec.num_heads, spec.num_kv_heads, spec.head_dim, spec.value_dim
+        if spec.mask not in ("window", "block"):
+            raise UnsupportedError(f"a mask of kind {spec.mask!r} (window or block)")
+        if spec.qk_gain and spec.qk_unit_eps is None:
+            raise UnsupportedError("a gain on q and k that are not divided by their root mean square")
         if H < 1 or G < 1 or H % G:
             raise UnsupportedError(f"{H} query heads over {G} key heads, which do not group evenly")
         unit = 1 if dtype == torch.float32 else 16       # the bfloat16 attention kernels take head sizes in 16s
@@ -76,7 +85,12 @@ class SinkAttention:
         self.H, self.G, self.D, self.V = H, G, D, V
         self.scale = float(spec.scale) if spec.scale is not None else 1.0 / math.sqrt(D)
         self.window = int(spec.window or 0)
-        self.proj = Linear.fused([params["q"], params["k"], params["v"]])
+        # what the attention kernels are told: a window as it is, blocks of positions as a negative number
+        self.mask = -self.window if spec.mask == "block" else self.window
+        biases = [params["q.b"], params["k.b"], params["v.b"]] if spec.qkv_bias else None
+        self.proj = Linear.fused([params["q"], params["k"], params["v"]], biases)
+        self.q_gain = params["q.norm"].to(torch.float32).contiguous() if spec.qk_gain else None
+        self.k_gain = params["k.norm"].to(torch.float32).contiguous() if spec.qk_gain else None
         self.sinks = head_sinks(spec.sink, H, params, device)
         self.slopes = head_slopes(spec.distance_slopes, H, float(spec.slope_span), device)
         self.temperature = ((float(spec.temperature_coef), int(spec.temperature_every))
@@ -89,6 +103,7 @@ class SinkAttention:
         self.o_proj = Linear(w_o)
 
     def cache_spec(self):
+        # (no key further back than the block's size is ever read: pages behind it come back as behind a window)
         return KVCacheSpec(self.G, self.padded, self.window or None)
 
     def state_spec(self):
@@ -102,9 +117,10 @@ class SinkAttention:
         n = rows.shape[0]
         q = torch.empty((n, self.H * self.padded), dtype=self.dtype, device=rows.device)
         kernels.head_prepare(rows, 0, batch, kv, q, self.H, self.G, self.D, self.V, self.padded,
-                             unit_eps=self.spec.qk_unit_eps, temperature=self.temperature, write_kv=ctx.writes_cache)
+                             unit_eps=self.spec.qk_unit_eps, q_gain=self.q_gain, k_gain=self.k_gain,
+                             temperature=self.temperature, write_kv=ctx.writes_cache)
         out = torch.empty((n, self.H * self.padded), dtype=self.dtype, device=rows.device)
-        kernels.sink_attention(q, out, batch, kv, self.H, self.G, self.padded, self.scale, self.window,
+        kernels.sink_attention(q, out, batch, kv, self.H, self.G, self.padded, self.scale, self.mask,
                                sinks=self.sinks, slopes=self.slopes)
         return self.o_proj.forward(out, out_dtype=torch.float32, add_into=getattr(ctx, "residual", None))
 

@@ -7,7 +7,7 @@ import torch
 from .. import kernels
 from ..errors import ConfigError
 from ..weights.loader import ParamDecl
-from .registry import NORMS, lookup, register_embed_transform, register_logit_transform
+from .registry import NORMS, lookup, register_embed_transform, register_final_transform, register_logit_transform
 
 
 class EmbeddingScale:
@@ -82,3 +82,48 @@ class LogitScale:
 register_embed_transform("learned_position", LearnedPosition)
 register_embed_transform("stream_norm", StreamNorm)
 register_logit_transform("scale", LogitScale)
+
+
+class StreamCopies:
+    """The stream behind the embedding ``extra["stream_copies"]`` times, [rows, copies * width]: what layers over
+    several copies of the stream start from."""
+
+    graph_safe = True
+
+    def __init__(self, spec, params: dict, dtype, device):
+        self.copies = int(spec.extra["stream_copies"])
+
+    def __call__(self, x, batch):
+        return kernels.stream_copies(x, self.copies)
+
+
+class StreamCopiesSum:
+    """Before the final norm: the sum of the copies of the stream, for the rows whose logits are wanted."""
+
+    graph_safe = True
+
+    def __init__(self, spec, params: dict, dtype, device):
+        self.copies = int(spec.extra["stream_copies"])
+        self.ones = torch.ones((self.copies,), dtype=torch.float32, device=device)
+
+    def __call__(self, x, batch):
+        return kernels.hc_step(x, self.copies, read=self.ones, rows=batch.logit_rows)
+
+
+class LogitSoftcap:
+    """logits <- cap * tanh(logits / cap), cap = extra["logit_softcap"]."""
+
+    graph_safe = True
+
+    def __init__(self, spec, params: dict, dtype, device):
+        self.cap = float(spec.extra["logit_softcap"])
+        if not self.cap > 0:
+            raise ConfigError(f"a soft cap of {self.cap} on the logits")
+
+    def __call__(self, logits, batch):
+        return kernels.softcap_(logits, self.cap) if logits.numel() else logits
+
+
+register_embed_transform("stream_copies", StreamCopies)
+register_final_transform("stream_copies_sum", StreamCopiesSum)
+register_logit_transform("softcap", LogitSoftcap)

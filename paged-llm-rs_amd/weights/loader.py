@@ -33,8 +33,10 @@ from .safetensors_io import SafetensorsFile
 
 @dataclass(frozen=True)
 class ParamDecl:
-    """One tensor a part needs.  ``role`` is ``matrix``, ``embedding``, ``gain`` or
-    ``bias``; it picks the random initialisation and nothing else."""
+    """One tensor a part needs.  ``role`` is ``matrix``, ``embedding``, ``gain``, ``bias``, the weights of several
+    copies of the stream (``copy_in``, ``copy_out``, ``copy_mix``), a gain stored around zero (``gain_around_zero``)
+    or a table of ``top`` out of n choices a row (``choice_table:<n>``, integers); it picks the random
+    initialisation and nothing else."""
     name: str
     shape: tuple
     role: str = "matrix"

@@ -35,9 +35,24 @@ def random_tensor(name: str, shape, role: str, seed: int, std: float, gain_std: 
                   dtype: torch.dtype) -> torch.Tensor:
     g = torch.Generator(device="cpu")
     g.manual_seed(_tensor_seed(seed, name))
+    if role.startswith("choice_table:"):
+        # a row names ``shape[1]`` different experts of the ``choice_table:<count>`` there are
+        count = int(role.split(":", 1)[1])
+        order = torch.rand((shape[0], count), generator=g).argsort(dim=1)
+        return order[:, :shape[1]].to(torch.int32).contiguous()
     x = torch.randn(tuple(shape), generator=g, dtype=torch.float32)
     if role == "gain":
         x = 1.0 + x * gain_std
+    elif role == "gain_around_zero":
+        x = x * gain_std
+    elif role == "copy_in":
+        # weights with which the copies of the stream are read: around an even share each
+        x = (1.0 + x * gain_std) / shape[0]
+    elif role == "copy_out":
+        x = 1.0 + x * gain_std
+    elif role == "copy_mix":
+        # how the copies are rebuilt from each other: around keeping each as it is
+        x = torch.eye(shape[0]) + x * gain_std * 0.5
     else:
         x = x * std
     return x.to(dtype)
@@ -65,7 +80,7 @@ def write_random_model(out_dir, config, seed: int = 0, std: float = 0.02, gain_s
     out_dir.mkdir(parents=True, exist_ok=True)
     (out_dir / "config.json").write_text(json.dumps(config_dict, indent=2) + "\n")
     items = [
-        (d.name, tuple(d.shape), torch_dtype,
+        (d.name, tuple(d.shape), torch.int32 if d.role.startswith("choice_table:") else torch_dtype,
          (lambda d=d: random_tensor(d.name, d.shape, d.role, seed, std, gain_std, torch_dtype)))
         for d in decls
     ]
