@@ -324,7 +324,30 @@ def lefavik_config(width: int, ff: int, heads: int, layers: int, vocab: int) -> 
             "logit_scale": 1.0, "max_positions": 8192, "layers": chosen}
 
 
-DESIGNS = {"papivik": papivik_config, "lefavik": lefavik_config}
+# --only mukenex: the Mukenex design (four copies of the stream; layers of linear attention with fixed decays, of
+# windowed attention over one small vector a token with a gate an element, and of grouped attention inside blocks of
+# positions, the first with a dense feed-forward, the others with eight experts of which a table names a token's two,
+# each half the dense width, so that a token multiplies as much as in the dense model; a soft cap on the logits) at the
+# same sizes, beside Qwen3 dense and beside Lefavik, the design whose layers are the nearest to these.
+def mukenex_config(width: int, ff: int, heads: int, layers: int, vocab: int) -> dict:
+    experts = {"kind": "moe", "expert": {"ff": ff // 2}, "router": {"experts": 8, "top": 2}}
+    kinds = [
+        {"type": "lightning", "mixer": {"heads": heads // 2, "dim": 128, "vdim": 128,
+                                        "decay": [1.0 - 2.0 ** (-5 - 3 * h / max(heads // 2 - 1, 1)) for h in range(heads // 2)]},
+         "mlp": {"kind": "dense", "ff": ff}},
+        {"type": "latent_attention", "mixer": {"heads": heads, "dim": 64, "rot_dim": 64, "vdim": 128, "kv_rank": 192,
+                                               "scale": 128 ** -0.5, "rot": {"dims": 64, "base": 1000000.0},
+                                               "mask": {"size": 512}}, "mlp": experts},
+        {"type": "attention", "mixer": {"heads": heads, "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                                        "mask": {"size": 512}}, "mlp": experts},
+    ]
+    return {"architecture": "Mukenex", "norm": {"eps": 1e-6}, "vocab": vocab, "width": width, "streams": 4,
+            "logit_softcap": 30.0, "layers": [kinds[i % 3] for i in range(layers)]}
+
+
+DESIGNS = {"papivik": papivik_config, "lefavik": lefavik_config, "mukenex": mukenex_config}
+# the models a design is measured beside, after Qwen3 dense
+BESIDE = {"mukenex": ("lefavik",)}
 
 
 def papivik_table(torch, args, design: str = "papivik") -> int:
@@ -343,7 +366,8 @@ def papivik_table(torch, args, design: str = "papivik") -> int:
             continue
         vocab = COMMON["vocab_size"]
         qwen = dict(SHAPES[beside][1], num_hidden_layers=layers, tie_word_embeddings=False)
-        for name, config in ((design, DESIGNS[design](width, ff, heads, layers, vocab)), ("qwen3", qwen)):
+        others = tuple((other, DESIGNS[other](width, ff, heads, layers, vocab)) for other in BESIDE.get(design, ()))
+        for name, config in ((design, DESIGNS[design](width, ff, heads, layers, vocab)), ("qwen3", qwen)) + others:
             with tempfile.TemporaryDirectory() as tmp:
                 say(f"{size}: writing and loading a random {layers}-layer {name} model of width {width}")
                 folder = write_random_model(Path(tmp) / "model", config, seed=0, std=0.02, gain_std=0.1, dtype="bfloat16")
@@ -454,8 +478,8 @@ def main() -> int:
     parser.add_argument("--ahead", choices=["on", "off"], default="on",
                         help="--only engine: whether the engine queues a decoding step before it has read the tokens "
                              "of the one before")
-    parser.add_argument("--size", choices=sorted(PAPIVIK_SIZES), default=None, help="--only papivik or lefavik: one of the sizes alone")
-    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving", "products", "papivik", "lefavik"], default=None,
+    parser.add_argument("--size", choices=sorted(PAPIVIK_SIZES), default=None, help="--only papivik, lefavik or mukenex: one of the sizes alone")
+    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving", "products", "papivik", "lefavik", "mukenex"], default=None,
                         help="run one part alone: the decode steps at --batch, the prefill, or (not part of the "
                              "default line) the whole engine on 1/4/16/32/64/128 requests at once, 16 prompt tokens and "
                              "128 generated each, as the reference's own table of clients does; mixed: one step of a "
@@ -465,7 +489,8 @@ def main() -> int:
                              "products: the layer products of the 8B and 32B shapes at 8 to 64 rows, weights from memory, "
                              "by the library and by the two hand-written products of few rows; papivik: prefill and decode "
                              "of the Papivik design at layer sizes of the 0.6B and 8B shapes beside Qwen3 dense of the same "
-                             "width, layers and vocabulary; lefavik: the same for the Lefavik design")
+                             "width, layers and vocabulary; lefavik: the same for the Lefavik design; mukenex: the same for the Mukenex "
+                             "design, beside Lefavik too")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU; this engine has no multi-GPU path (N must be 1)")
