@@ -30,6 +30,17 @@ typedef float gt_f32x2 __attribute__((ext_vector_type(2)));
 #define GT_STORE 0
 #define GT_SWIGLU 1
 #define GT_ADD 2
+#define GT_STORE32 3       // y is 32-bit and takes the result as it is (grouped products only)
+
+// Grouped: the rows are dealt to groups (experts), every group with a weight matrix of its own, one behind the
+// other in w.  A tile of 128 rows belongs to one group (`tile_group`, negative: a tile nobody uses); row r of
+// the tile reads row gather[r] of x (null: row r itself; negative: a row of padding, which reads row 0 and
+// whose result nobody looks at) and writes row r of y.  Output columns past N are not written (N a multiple of 4).
+struct GtGroups {
+    const int* tile_group;     // [row tiles]
+    const int* gather;         // [row tiles * 128] or null
+    long long w_stride;        // elements between two groups' matrices
+};
 
 // 16 bytes a lane from global memory straight into LDS (see attention_prefill.hip: assembly, so that
 // the compiler does not count the load and make every later read of LDS wait for all of them).
@@ -46,10 +57,10 @@ __device__ __forceinline__ uint32_t gt_pack2(float lo, float hi) {
 // EPI: GT_STORE y = result (bfloat16).  GT_SWIGLU: w is [gate rows | up rows], N counts the gate rows, and
 // y = silu(gate) * up (bfloat16).  GT_ADD: y is the 32-bit residual stream and takes the result.
 // M any; N a multiple of 128 (64 for SwiGLU); K a multiple of 32.
-template <int EPI>
+template <int EPI, bool GROUPED = false>
 __global__ void __launch_bounds__(256, 2)
 gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ y_, int M, int N, int K,
-                  int row_tiles, int total, int act) {
+                  int row_tiles, int total, int act, GtGroups groups) {
     extern __shared__ __attribute__((aligned(16))) uint16_t gt_lds[];   // [stage][x rows 0..127 | w rows 0..127][32]
 
     // Workgroups are dealt round-robin to the eight XCDs; consecutive tiles (the row tiles of one column
@@ -60,6 +71,11 @@ gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, vo
     const int col_tile = work / row_tiles;
     constexpr int COLS = EPI == GT_SWIGLU ? GT_BN / 2 : GT_BN;   // output columns a workgroup
     const int n0 = col_tile * COLS;
+    if constexpr (GROUPED) {
+        const int group = groups.tile_group[m0 / GT_BM];
+        if (group < 0) return;                       // (the whole workgroup)
+        w += static_cast<long long>(group) * groups.w_stride;
+    }
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -78,10 +94,15 @@ gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, vo
         size_t grow;
         if (chunk < 8) {
             grow = static_cast<size_t>(min(m0 + row, M - 1));
+            if constexpr (GROUPED) {
+                if (groups.gather != nullptr) grow = static_cast<size_t>(max(groups.gather[m0 + row], 0));
+            }
             from[i] = reinterpret_cast<const char*>(x) + (grow * K + piece * 8) * 2;
         } else {
             // SwiGLU: rows 0..63 of the tile are gate rows n0.., rows 64..127 the up rows N + n0..
-            grow = EPI == GT_SWIGLU ? static_cast<size_t>(row < 64 ? n0 + row : N + n0 + row - 64) : static_cast<size_t>(n0 + row);
+            // (grouped, the last tile of columns may reach past N: it reads the last row again)
+            const int wr = GROUPED ? min(n0 + (EPI == GT_SWIGLU ? row & 63 : row), N - 1) - n0 : (EPI == GT_SWIGLU ? row & 63 : row);
+            grow = EPI == GT_SWIGLU ? static_cast<size_t>(row < 64 ? n0 + wr : N + n0 + wr) : static_cast<size_t>(n0 + wr);
             from[i] = reinterpret_cast<const char*>(w) + (grow * K + piece * 8) * 2;
         }
         lds_chunk[i] = chunk * 16 * GT_BK;           // elements from the stage's start
@@ -176,7 +197,7 @@ gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, vo
     // acc[t][mb][4 j + i]: output column (of the wave's 32 of half t) 8 j + 4 h + i, row 64 wm + 32 mb + r32
     __syncthreads();                                 // every wave has read its last operands
     constexpr int OUT_COLS = EPI == GT_SWIGLU ? GT_BN / 2 : GT_BN;
-    constexpr int OUT_BYTES = EPI == GT_ADD ? 4 : 2;
+    constexpr int OUT_BYTES = (EPI == GT_ADD || EPI == GT_STORE32) ? 4 : 2;
     constexpr int PITCH = OUT_COLS * OUT_BYTES + 16;      // bytes (a multiple of 16: rows are read 16 bytes a lane)
     char* staged = reinterpret_cast<char*>(gt_lds);
 #pragma unroll
@@ -202,7 +223,7 @@ gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, vo
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int col = 64 * wn + 32 * t + 4 * h + 8 * j;
-                    if constexpr (EPI == GT_ADD) {
+                    if constexpr (EPI == GT_ADD || EPI == GT_STORE32) {
                         gt_f32x4 v;
 #pragma unroll
                         for (int i = 0; i < 4; ++i) v[i] = acc[t][mb][4 * j + i];
@@ -223,7 +244,10 @@ gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, vo
 #pragma unroll 4
     for (int r = tid / LANES_A_ROW; r < GT_BM; r += ROWS_A_PASS) {
         const int row = m0 + r;
-        if (row >= M) break;
+        if (!GROUPED && row >= M) break;             // (grouped, y has every tile's rows)
+        if constexpr (GROUPED) {
+            if (n0 + (piece + 1) * (16 / OUT_BYTES) > N) continue;      // columns past the matrix
+        }
         const gt_f32x4 got = *reinterpret_cast<const gt_f32x4*>(staged + r * PITCH + piece * 16);
         char* out = static_cast<char*>(y_) + (static_cast<size_t>(row) * N + n0) * OUT_BYTES + piece * 16;
         if constexpr (EPI == GT_ADD) {
@@ -238,13 +262,18 @@ gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, vo
 }
 
 template <int EPI>
+constexpr size_t gt_out_bytes() {
+    return static_cast<size_t>(GT_BM) * ((EPI == GT_ADD || EPI == GT_STORE32) ? GT_BN * 4 + 16 : (EPI == GT_SWIGLU ? GT_BN + 16 : GT_BN * 2 + 16));
+}
+
+template <int EPI>
 static int gt_launch(const void* x, const void* w, void* y, int M, int N, int K, int act, hipStream_t stream) {
     constexpr int COLS = EPI == GT_SWIGLU ? GT_BN / 2 : GT_BN;
     const int row_tiles = pl_ceil_div(M, GT_BM);
     const long long total = static_cast<long long>(row_tiles) * (N / COLS);
     PL_REQUIRE(total > 0 && total < (1ll << 30), "tiled product: %lld workgroups", total);
     // the stages of operands, or the tile on its way out (32-bit rows of 128 with their pitch), whichever is more
-    constexpr size_t out_bytes = static_cast<size_t>(GT_BM) * (EPI == GT_ADD ? GT_BN * 4 + 16 : (EPI == GT_SWIGLU ? GT_BN + 16 : GT_BN * 2 + 16));
+    constexpr size_t out_bytes = gt_out_bytes<EPI>();
     constexpr size_t stage_bytes = static_cast<size_t>(GT_STAGES) * GT_STAGE_ELEMS * 2;
     const size_t lds_bytes = out_bytes > stage_bytes ? out_bytes : stage_bytes;
     static bool raised = false;
@@ -255,8 +284,53 @@ static int gt_launch(const void* x, const void* w, void* y, int M, int N, int K,
         raised = true;
     }
     gemm_tiled_kernel<EPI><<<static_cast<int>(total), 256, lds_bytes, stream>>>(
-        static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y, M, N, K, row_tiles, static_cast<int>(total), act);
+        static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y, M, N, K, row_tiles, static_cast<int>(total), act,
+        GtGroups{nullptr, nullptr, 0});
     PL_CHECK_LAUNCH("gemm_tiled");
+    return 0;
+}
+
+template <int EPI>
+static int gt_launch_grouped(const void* x, const void* w, void* y, int row_tiles, int N, int K, int act, GtGroups groups,
+                             int x_rows, hipStream_t stream) {
+    constexpr int COLS = EPI == GT_SWIGLU ? GT_BN / 2 : GT_BN;
+    const long long total = static_cast<long long>(row_tiles) * pl_ceil_div(N, COLS);
+    PL_REQUIRE(total > 0 && total < (1ll << 30), "grouped tiled product: %lld workgroups", total);
+    constexpr size_t out_bytes = gt_out_bytes<EPI>();
+    constexpr size_t stage_bytes = static_cast<size_t>(GT_STAGES) * GT_STAGE_ELEMS * 2;
+    const size_t lds_bytes = out_bytes > stage_bytes ? out_bytes : stage_bytes;
+    static bool raised = false;
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiled_kernel<EPI, true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+        PL_REQUIRE(e == hipSuccess, "grouped tiled product: %zu bytes of LDS refused: %s", lds_bytes, hipGetErrorString(e));
+        raised = true;
+    }
+    // (M: the rows of x that exist when rows are read in place, the tiles' rows otherwise)
+    gemm_tiled_kernel<EPI, true><<<static_cast<int>(total), 256, lds_bytes, stream>>>(
+        static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y, x_rows, N, K, row_tiles, static_cast<int>(total), act,
+        groups);
+    PL_CHECK_LAUNCH("gemm_tiled_grouped");
+    return 0;
+}
+
+// The product over rows dealt to groups, every group against a matrix of its own (see GtGroups).
+// x: bfloat16 [x_rows, K], read through `gather` ([row_tiles * 128] row numbers, negative: padding) or, with gather
+// null, in place (x_rows >= row_tiles * 128).  w: bfloat16, group g's matrix at w + g * w_stride: [N, K], or
+// [2 N, K] with the gate rows first for epilogue 1.  y: [row_tiles * 128, N], bfloat16 for epilogues 0 and 1
+// (1: act(gate) * up), 32-bit for epilogue 3.  K a multiple of 32, N of 8 (of 64 for epilogue 1).
+extern "C" int pl_gemm_tiled_grouped(const void* x, const void* w, void* y, const int* tile_group, const int* gather,
+                                     long long w_stride, int row_tiles, int x_rows, int N, int K, int epilogue, int act,
+                                     hipStream_t stream) {
+    PL_REQUIRE(act >= PL_ACT_SILU && act <= PL_ACT_GELU, "grouped tiled product: activation code %d", act);
+    PL_REQUIRE(row_tiles > 0 && x_rows > 0 && N > 0 && K > 0 && K % GT_BK == 0 && N % 8 == 0 && (epilogue != GT_SWIGLU || N % (GT_BN / 2) == 0),
+               "grouped tiled product: %d tiles of rows, %d columns, inner width %d, epilogue %d", row_tiles, N, K, epilogue);
+    PL_REQUIRE(tile_group != nullptr && (gather != nullptr || x_rows >= row_tiles * GT_BM), "grouped tiled product: %d rows for %d tiles", x_rows, row_tiles);
+    const GtGroups groups{tile_group, gather, w_stride};
+    if (epilogue == GT_SWIGLU) return gt_launch_grouped<GT_SWIGLU>(x, w, y, row_tiles, N, K, act, groups, x_rows, stream);
+    if (epilogue == GT_STORE32) return gt_launch_grouped<GT_STORE32>(x, w, y, row_tiles, N, K, act, groups, x_rows, stream);
+    if (epilogue == GT_STORE) return gt_launch_grouped<GT_STORE>(x, w, y, row_tiles, N, K, act, groups, x_rows, stream);
+    PL_REQUIRE(false, "grouped tiled product: epilogue %d", epilogue);
     return 0;
 }
 

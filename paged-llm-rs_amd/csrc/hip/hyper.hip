@@ -7,8 +7,12 @@
 // may be left out.  Sums, statistic and gain are 32-bit; the normed row is rounded once, when stored.
 //
 // Experts by table.  Row t uses the `top` experts that table[id of t] names, each weighted 1/top; an
-// expert is down(act(gate x) * (up x)).  The kernels here serve few rows, a workgroup a (row, choice):
-// a row reads only its own experts' weights.
+// expert is down(act(gate x) * (up x)).  Two ways.  moe_rows, a workgroup a (row, choice): a row reads its
+// own experts' weights, in any type and size (the 32-bit path, and shapes the matrix cores' tiles do not
+// take).  moe_sort and moe_combine around the grouped tiled product (gemm_tiled.hip): the step's (row,
+// choice) pairs are dealt to their experts, every expert's pairs in tiles of 128 rows, so that an expert's
+// weights are read once a tile and multiplied on the matrix cores; a pair's result does not depend on which
+// other pairs share its tile.
 #include "common.hpp"
 
 #define HC_MAX_COPIES 8
@@ -273,5 +277,100 @@ extern "C" int pl_moe_rows(const void* x, const int* ids, const int* src, const 
         PL_REQUIRE(false, "moe_rows: dtype code %d", dtype);
     }
     PL_CHECK_LAUNCH("moe_rows");
+    return 0;
+}
+
+// ---- experts by table, the pairs dealt to their experts ---------------------------------------------------------
+
+// One workgroup.  Pair p = t * top + c (row t, its c-th expert).  Expert e's pairs get the slots
+// base[e] .. base[e] + count[e] - 1, base[e] a multiple of `tile`; gather[slot] = t (or -1 for the slots
+// between the experts' stretches), slot_of[p] = slot (or -1 for a pair of a padding row),
+// tile_group[i] = the expert of tile i (or -1 behind the last).  Which of an expert's pairs gets which of
+// its slots is left to the order in which the threads arrive: nothing computed from a slot depends on it.
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* ids, const int* src, const int* fed, const int* positions,
+                                                        const int* table, int n, int top, int E, int vocab, int tile,
+                                                        int tiles, int* gather, int* slot_of, int* tile_group) {
+    extern __shared__ int moe_counts[];               // count [E], base [E], cursor [E]
+    int* count = moe_counts;
+    int* base = moe_counts + E;
+    int* cursor = moe_counts + 2 * E;
+    for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = cursor[e] = 0;
+    for (int s = threadIdx.x; s < tiles * tile; s += blockDim.x) gather[s] = -1;
+    __syncthreads();
+    const int pairs = n * top;
+    auto expert_of = [&](int p) -> int {
+        const int t = p / top;
+        if (positions[t] < 0) return -1;
+        const int id = moe_token(ids, src, fed, t);
+        if (id < 0 || id >= vocab) return -1;
+        const int e = table[static_cast<size_t>(id) * top + (p - t * top)];
+        return (e >= 0 && e < E) ? e : -1;
+    };
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+        const int e = expert_of(p);
+        if (e >= 0) atomicAdd(&count[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0;                                   // in tiles
+        for (int e = 0; e < E; ++e) {
+            base[e] = at * tile;
+            const int mine = (count[e] + tile - 1) / tile;
+            for (int i = 0; i < mine && at + i < tiles; ++i) tile_group[at + i] = e;
+            at += mine;
+        }
+        for (; at < tiles; ++at) tile_group[at] = -1;
+    }
+    __syncthreads();
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+        const int e = expert_of(p);
+        int slot = -1;
+        if (e >= 0) {
+            slot = base[e] + atomicAdd(&cursor[e], 1);
+            gather[slot] = p / top;
+        }
+        slot_of[p] = slot;
+    }
+}
+
+// tiles: what the caller has room for, at least ceil(n * top / tile) + min(E, n * top).
+extern "C" int pl_moe_sort(const int* ids, const int* src, const int* fed, const int* positions, const int* table, int n,
+                           int top, int E, int vocab, int tile, int tiles, int* gather, int* slot_of, int* tile_group,
+                           hipStream_t stream) {
+    PL_REQUIRE(n > 0 && top > 0 && E > 0 && E <= 4096 && top <= E && vocab > 0 && tile > 0, "moe_sort: %d rows, %d of %d experts", n, top, E);
+    PL_REQUIRE(static_cast<long long>(n) * top < (1ll << 30) && tiles >= (n * top + tile - 1) / tile + (E < n * top ? E : n * top),
+               "moe_sort: %d tiles of %d for %d rows with %d of %d experts", tiles, tile, n, top, E);
+    PL_REQUIRE((src == nullptr) == (fed == nullptr), "moe_sort: rows fed from the step before need both the rows and the tokens");
+    moe_sort_kernel<<<1, 1024, 3 * E * sizeof(int), stream>>>(ids, src, fed, positions, table, n, top, E, vocab, tile, tiles,
+                                                               gather, slot_of, tile_group);
+    PL_CHECK_LAUNCH("moe_sort");
+    return 0;
+}
+
+// out[t, :] = (1/top) sum over c of y[slot_of[t * top + c], :], the choices in their order; a pair without a slot adds nothing.
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ slot_of,
+                                                          float* __restrict__ out, int top, int W) {
+    const int t = blockIdx.x;
+    const float share = 1.f / static_cast<float>(top);
+    for (int w = threadIdx.x * 4; w < W; w += blockDim.x * 4) {
+        float4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int c = 0; c < top; ++c) {
+            const int slot = slot_of[t * top + c];
+            if (slot < 0) continue;
+            const float4 v = *reinterpret_cast<const float4*>(y + static_cast<size_t>(slot) * W + w);
+            sum.x += v.x * share;
+            sum.y += v.y * share;
+            sum.z += v.z * share;
+            sum.w += v.w * share;
+        }
+        *reinterpret_cast<float4*>(out + static_cast<size_t>(t) * W + w) = sum;
+    }
+}
+
+extern "C" int pl_moe_combine(const float* y, const int* slot_of, float* out, int n, int top, int W, hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && top > 0 && W > 0 && W % 4 == 0, "moe_combine: %d rows of %d, %d a row", n, W, top);
+    if (n == 0) return 0;
+    moe_combine_kernel<<<n, 256, 0, stream>>>(y, slot_of, out, top, W);
+    PL_CHECK_LAUNCH("moe_combine");
     return 0;
 }

@@ -79,6 +79,9 @@ def _signatures(lib) -> None:
         "pl_stream_copies": [p, p, i, i, i, p],
         "pl_softcap": [p, f, ctypes.c_long, p],
         "pl_moe_rows": [p, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, p],
+        "pl_moe_sort": [p, p, p, p, p, i, i, i, i, i, i, p, p, p, p],
+        "pl_moe_combine": [p, p, p, i, i, i, p],
+        "pl_gemm_tiled_grouped": [p, p, p, p, p, ctypes.c_longlong, i, i, i, i, i, i, p],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name)
@@ -1549,4 +1552,52 @@ def moe_rows(x: torch.Tensor, batch, table: torch.Tensor, w_gate_up: torch.Tenso
                                  batch.positions.data_ptr(), table.data_ptr(), w_gate_up.data_ptr(), w_down.data_ptr(),
                                  h.data_ptr(), out.data_ptr(), _code(x, "rows"), n, W, F, E, top, vocab,
                                  activation_code(activation), _stream()))
+    return out
+
+
+MOE_TILE = 128       # rows of a tile of the grouped product
+
+
+def moe_grouped_applies(x: torch.Tensor, width: int, ff: int) -> bool:
+    """Whether the experts of a step run as grouped products on the matrix cores: bfloat16, an inner width the
+    tiles take (a multiple of 32), an expert width that is a multiple of 64."""
+    return x.dtype == torch.bfloat16 and width % 32 == 0 and ff % 64 == 0 and _attention_mode == "kernel"
+
+
+def moe_grouped(x: torch.Tensor, batch, table: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
+                activation: str = "silu") -> torch.Tensor:
+    """What ``moe_rows`` computes, with the step's (row, choice) pairs dealt to their experts first: an expert's
+    pairs fill tiles of 128 rows, and two grouped products on the matrix cores (gate and up with the activation
+    behind them; down with 32-bit sums out) read an expert's weights once a tile.  A last pass adds a row's
+    choices in their order, in 32-bit.  Nothing is read back by the host: the tiles are laid out for the most
+    a step of so many rows can need."""
+    n, W = x.shape
+    _need(x, "rows", None, torch.bfloat16)
+    E, F2, _ = w_gate_up.shape
+    F = F2 // 2
+    _need(w_gate_up, "gate and up weights of the experts", (E, 2 * F, W), x.dtype)
+    _need(w_down, "down weights of the experts", (E, W, F), x.dtype)
+    _need(table, "table of experts", None, torch.int32)
+    vocab, top = table.shape
+    out = torch.empty((n, W), dtype=torch.float32, device=x.device)
+    if n == 0:
+        return out
+    fed = getattr(batch, "fed_tokens", None)
+    src = batch.token_src if fed is not None else None
+    pairs = n * top
+    # every expert that has pairs may leave its last tile part empty
+    tiles = -(-pairs // MOE_TILE) + min(E, pairs)
+    slots = tiles * MOE_TILE
+    lib, stream = library(), _stream()
+    ints = torch.empty((slots + pairs + tiles,), dtype=torch.int32, device=x.device)
+    gather, slot_of, tile_group = ints[:slots], ints[slots:slots + pairs], ints[slots + pairs:]
+    _check(lib.pl_moe_sort(batch.token_ids.data_ptr(), _ptr(src), _ptr(fed), batch.positions.data_ptr(), table.data_ptr(),
+                           n, top, E, vocab, MOE_TILE, tiles, gather.data_ptr(), slot_of.data_ptr(), tile_group.data_ptr(), stream))
+    hidden = torch.empty((slots, F), dtype=torch.bfloat16, device=x.device)
+    _check(lib.pl_gemm_tiled_grouped(x.data_ptr(), w_gate_up.data_ptr(), hidden.data_ptr(), tile_group.data_ptr(),
+                                     gather.data_ptr(), 2 * F * W, tiles, n, F, W, 1, activation_code(activation), stream))
+    y = torch.empty((slots, W), dtype=torch.float32, device=x.device)
+    _check(lib.pl_gemm_tiled_grouped(hidden.data_ptr(), w_down.data_ptr(), y.data_ptr(), tile_group.data_ptr(), 0,
+                                     W * F, tiles, slots, W, F, 3, 0, stream))
+    _check(lib.pl_moe_combine(y.data_ptr(), slot_of.data_ptr(), out.data_ptr(), n, top, W, stream))
     return out

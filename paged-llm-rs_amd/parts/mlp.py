@@ -138,6 +138,8 @@ class TableExperts:
         self.table = table.contiguous()
 
     def forward(self, x, batch):
+        if kernels.moe_grouped_applies(x, x.shape[1], self.spec.intermediate_size):
+            return kernels.moe_grouped(x, batch, self.table, self.w_gate_up, self.w_down, self.activation)
         return kernels.moe_rows(x, batch, self.table, self.w_gate_up, self.w_down, self.activation)
 
 

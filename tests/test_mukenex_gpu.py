@@ -183,6 +183,45 @@ def test_experts_by_table(dtype, experts, top, ff, width, rows):
         assert torch.equal(fed, again)
 
 
+@pytest.mark.parametrize("experts,top,ff,width,rows", [(8, 2, 64, 192, 50), (8, 2, 64, 192, 1), (16, 4, 128, 256, 300), (32, 4, 128, 1024, 700),
+                                                      (4, 1, 256, 512, 129), (64, 8, 64, 96, 5), (3, 3, 192, 160, 1000), (2, 2, 1536, 1024, 64)])
+def test_experts_by_table_dealt_to_their_experts(experts, top, ff, width, rows):
+    """The grouped products on the matrix cores against the kernel that takes a row at a time (bfloat16): the same
+    pairs, the same weights, sums in another order.  Rows of padding give zeros; ids left on the device are taken;
+    an expert that nobody chose, experts with more than a tile of rows, more experts than pairs."""
+    from paged_llm_rs_amd import kernels
+
+    g = torch.Generator().manual_seed(experts * 100 + rows)
+    vocab = 53
+    w_gu = (torch.randn((experts, 2 * ff, width), generator=g) * width ** -0.5).to(torch.bfloat16).cuda()
+    w_down = (torch.randn((experts, width, ff), generator=g) * ff ** -0.5).to(torch.bfloat16).cuda()
+    x = torch.randn((rows, width), generator=g).to(torch.bfloat16).cuda()
+    assert kernels.moe_grouped_applies(x, width, ff)
+    table = torch.rand((vocab, experts), generator=g).argsort(1)[:, :top].to(torch.int32)
+    if experts > 2:
+        table[table == 1] = 0 if top == 1 else table[table == 1]      # (with one choice a row, expert 1 is never chosen)
+    table = table.cuda()
+    ids = torch.randint(0, vocab, (rows,), generator=g).tolist()
+    positions = list(range(rows))
+    if rows > 2:
+        positions[rows // 2] = -1
+    batch = _Rows(ids, positions)
+    if rows >= 7:
+        batch.fed_tokens = torch.tensor([3, 40, 17], dtype=torch.int32).cuda()
+        src = [-1] * rows
+        src[1], src[4] = 2, 0
+        batch.token_src = torch.tensor(src, dtype=torch.int32).cuda()
+    want = kernels.moe_rows(x, batch, table, w_gu, w_down, "silu")
+    for _ in range(2):           # (which slot a pair gets may differ from run to run; what it computes may not)
+        got = kernels.moe_grouped(x, batch, table, w_gu, w_down, "silu")
+        assert got.shape == want.shape and torch.isfinite(got).all()
+        assert (got - want).abs().max() <= 1e-2 * want.abs().max()
+        if rows > 2:
+            assert float(got[rows // 2].abs().max()) == 0.0
+    again = kernels.moe_grouped(x, batch, table, w_gu, w_down, "silu")
+    assert torch.equal(got, again), "a row's result does not depend on its place in a tile"
+
+
 def _blocks_oracle(q, k, v, positions, block, scale):
     """Softmax attention of one request's queries at ``positions`` over keys 0 .. T - 1 inside the query's own block."""
     T = k.shape[0]
