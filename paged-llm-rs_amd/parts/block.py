@@ -295,6 +295,17 @@ class SharedNormBlock:
 register_block("shared_norm", SharedNormBlock)
 
 
+class PendingCopies:
+    """A rebuild of the copies of the stream that has not run yet: the last sublayer's output and its weights.  The
+    layer behind runs it in the pass that reads out its own first rows."""
+
+    __slots__ = ("y", "mix", "out")
+    filled = True            # (what a layer hands to the next is looked at only when it says it holds something)
+
+    def __init__(self, y, mix, out):
+        self.y, self.mix, self.out = y, mix, out
+
+
 class HyperConnectionBlock:
     """The pre-norm arrangement over several copies of the stream.  The stream a layer gets is [rows, S * width]:
     S copies x_1 .. x_S of every row, one behind the other.  A sublayer (1: the mixer, 2: the feed-forward, where
@@ -303,7 +314,9 @@ class HyperConnectionBlock:
     and the plain sums x <- x + y, computed as one copy with weights of one.
 
     Everything about the copies is 32-bit.  One kernel rebuilds the copies behind a sublayer and reads out the
-    next sublayer's normed rows in the same pass (``kernels.hc_step``).  Sublayers hand back 32-bit rows.
+    next sublayer's normed rows in the same pass (``kernels.hc_step``), also from one layer to the next: a layer
+    that is followed by another of this arrangement leaves its last rebuild to that layer's first pass
+    (``PendingCopies``), so a layer with a feed-forward is two passes over the copies.  Sublayers hand back 32-bit rows.
     Tensor names: the norms' gains under the norms' own names; ``hc1.in`` [S], ``hc1.out`` [S], ``hc1.mix`` [S, S]
     (from, to) for the mixer and ``hc2.*`` for the feed-forward."""
 
@@ -353,6 +366,7 @@ class HyperConnectionBlock:
         if not 1 <= self.copies <= kernels.HC_MAX_COPIES:
             raise ConfigError(f"{self.copies} copies of the stream (1 to {kernels.HC_MAX_COPIES})")
         self.norm1 = norm(layer.norm, hidden, {"weight": params[n["norm1"]]}, dtype, device)
+        self.norm1.takes_pending_copies = self.copies       # (how the layer before learns that its last rebuild can wait)
         self.mixer = lookup(MIXERS, layer.mixer.kind, "mixer")(
             layer.mixer, hidden, scoped(params, n["mixer"]), dtype, device, shared)
         self.weights1 = self._copy_weights(params, n["copies1"], layer.stream_copies, device)
@@ -375,6 +389,19 @@ class HyperConnectionBlock:
     def graph_safe(self) -> bool:
         return getattr(self.mixer, "graph_safe", True) and getattr(self.feed_forward, "graph_safe", True)
 
+    @property
+    def first_norm(self):
+        return self.norm1
+
+    def _finish(self, resid, y, mix, out, ctx):
+        """The layer's last rebuild: now, or, where the next layer is of this arrangement, in that layer's first pass."""
+        after = getattr(ctx, "norm_after", None)
+        if ctx.trace is None and after is not None and getattr(after, "takes_pending_copies", None) == self.copies:
+            ctx.handed_out = PendingCopies(y, mix, out)
+        else:
+            kernels.hc_step(resid, self.copies, y=y, mix=mix, out=out)
+        return None
+
     def _feed(self, rows, ctx):
         ffn = self.feed_forward
         if getattr(ffn, "takes_batch", False):
@@ -388,16 +415,19 @@ class HyperConnectionBlock:
             raise ConfigError(f"a stream of rows of {resid.shape[1]} for {self.copies} copies of {self.hidden}")
         S = self.copies
         in1, mix1, out1 = self.weights1
-        rows = kernels.hc_step(resid, S, read=in1, gain=self.norm1.gain32, eps=self.norm1.eps, read_dtype=self.dtype)
+        before = getattr(ctx, "handed", None)
+        if isinstance(before, PendingCopies):
+            rows = kernels.hc_step(resid, S, y=before.y, mix=before.mix, out=before.out, read=in1, gain=self.norm1.gain32,
+                                   eps=self.norm1.eps, read_dtype=self.dtype)
+        else:
+            rows = kernels.hc_step(resid, S, read=in1, gain=self.norm1.gain32, eps=self.norm1.eps, read_dtype=self.dtype)
         mixed = self.mixer.forward(rows, ctx)
         if self.feed_forward is None:
-            kernels.hc_step(resid, S, y=mixed, mix=mix1, out=out1)
-            return None
+            return self._finish(resid, mixed, mix1, out1, ctx)
         in2, mix2, out2 = self.weights2
         rows = kernels.hc_step(resid, S, y=mixed, mix=mix1, out=out1, read=in2, gain=self.norm2.gain32,
                                eps=self.norm2.eps, read_dtype=self.dtype)
-        kernels.hc_step(resid, S, y=self._feed(rows, ctx), mix=mix2, out=out2)
-        return None
+        return self._finish(resid, self._feed(rows, ctx), mix2, out2, ctx)
 
 
 register_block("hyper_connections", HyperConnectionBlock)
