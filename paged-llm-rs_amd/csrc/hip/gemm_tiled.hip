@@ -40,6 +40,11 @@ struct GtGroups {
     const int* tile_group;     // [row tiles]
     const int* gather;         // [row tiles * 128] or null
     long long w_stride;        // elements between two groups' matrices
+    // Few tiles of rows over a deep inner width leave most of the chip idle: the inner width is then cut into
+    // `splits` stretches, a launch has `splits` workgroups a tile, and stretch s leaves its sums in the s-th copy
+    // of y (`y_split_stride` elements apart); whoever reads y adds the copies in their order.
+    int splits;
+    long long y_split_stride;
 };
 
 // 16 bytes a lane from global memory straight into LDS (see attention_prefill.hip: assembly, so that
@@ -65,8 +70,13 @@ gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, vo
 
     // Workgroups are dealt round-robin to the eight XCDs; consecutive tiles (the row tiles of one column
     // tile first) go to one XCD, whose L2 then holds the rows of w they share.
-    int work = blockIdx.x;
-    if ((total & 7) == 0) work = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
+    int at = blockIdx.x, split = 0;
+    if constexpr (GROUPED) {
+        split = at / total;                          // (total: the workgroups of one stretch of the inner width)
+        at -= split * total;
+    }
+    int work = at;
+    if ((total & 7) == 0) work = (at & 7) * (total >> 3) + (at >> 3);
     const int m0 = (work % row_tiles) * GT_BM;
     const int col_tile = work / row_tiles;
     constexpr int COLS = EPI == GT_SWIGLU ? GT_BN / 2 : GT_BN;   // output columns a workgroup
@@ -107,7 +117,16 @@ gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, vo
         }
         lds_chunk[i] = chunk * 16 * GT_BK;           // elements from the stage's start
     }
-    const int steps = K / GT_BK;
+    int steps = K / GT_BK;
+    if constexpr (GROUPED) {
+        if (groups.splits > 1) {
+            const int first = split * steps / groups.splits, behind = (split + 1) * steps / groups.splits;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) from[i] += static_cast<size_t>(first) * GT_BK * 2;
+            steps = behind - first;
+            y_ = static_cast<char*>(y_) + static_cast<size_t>(split) * groups.y_split_stride * ((EPI == GT_ADD || EPI == GT_STORE32) ? 4 : 2);
+        }
+    }
     auto ask = [&](int step) {                       // past the end the last step is asked for again: the count of
         const int s = min(step, steps - 1);          // loads on their way stays the same for every step
         uint16_t* stage = gt_lds + (step % GT_STAGES) * GT_STAGE_ELEMS;
@@ -285,7 +304,7 @@ static int gt_launch(const void* x, const void* w, void* y, int M, int N, int K,
     }
     gemm_tiled_kernel<EPI><<<static_cast<int>(total), 256, lds_bytes, stream>>>(
         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y, M, N, K, row_tiles, static_cast<int>(total), act,
-        GtGroups{nullptr, nullptr, 0});
+        GtGroups{nullptr, nullptr, 0, 1, 0});
     PL_CHECK_LAUNCH("gemm_tiled");
     return 0;
 }
@@ -307,7 +326,7 @@ static int gt_launch_grouped(const void* x, const void* w, void* y, int row_tile
         raised = true;
     }
     // (M: the rows of x that exist when rows are read in place, the tiles' rows otherwise)
-    gemm_tiled_kernel<EPI, true><<<static_cast<int>(total), 256, lds_bytes, stream>>>(
+    gemm_tiled_kernel<EPI, true><<<static_cast<int>(total * groups.splits), 256, lds_bytes, stream>>>(
         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y, x_rows, N, K, row_tiles, static_cast<int>(total), act,
         groups);
     PL_CHECK_LAUNCH("gemm_tiled_grouped");
@@ -319,14 +338,17 @@ static int gt_launch_grouped(const void* x, const void* w, void* y, int row_tile
 // null, in place (x_rows >= row_tiles * 128).  w: bfloat16, group g's matrix at w + g * w_stride: [N, K], or
 // [2 N, K] with the gate rows first for epilogue 1.  y: [row_tiles * 128, N], bfloat16 for epilogues 0 and 1
 // (1: act(gate) * up), 32-bit for epilogue 3.  K a multiple of 32, N of 8 (of 64 for epilogue 1).
+// splits > 1 (epilogue 3 only): y has that many copies, [splits][row_tiles * 128, N], a stretch of K each.
 extern "C" int pl_gemm_tiled_grouped(const void* x, const void* w, void* y, const int* tile_group, const int* gather,
                                      long long w_stride, int row_tiles, int x_rows, int N, int K, int epilogue, int act,
-                                     hipStream_t stream) {
+                                     int splits, hipStream_t stream) {
+    PL_REQUIRE(splits >= 1 && splits <= K / GT_BK && (splits == 1 || epilogue == GT_STORE32),
+               "grouped tiled product: %d stretches of an inner width of %d, epilogue %d", splits, K, epilogue);
     PL_REQUIRE(act >= PL_ACT_SILU && act <= PL_ACT_GELU, "grouped tiled product: activation code %d", act);
     PL_REQUIRE(row_tiles > 0 && x_rows > 0 && N > 0 && K > 0 && K % GT_BK == 0 && N % 8 == 0 && (epilogue != GT_SWIGLU || N % (GT_BN / 2) == 0),
                "grouped tiled product: %d tiles of rows, %d columns, inner width %d, epilogue %d", row_tiles, N, K, epilogue);
     PL_REQUIRE(tile_group != nullptr && (gather != nullptr || x_rows >= row_tiles * GT_BM), "grouped tiled product: %d rows for %d tiles", x_rows, row_tiles);
-    const GtGroups groups{tile_group, gather, w_stride};
+    const GtGroups groups{tile_group, gather, w_stride, splits, static_cast<long long>(row_tiles) * GT_BM * N};
     if (epilogue == GT_SWIGLU) return gt_launch_grouped<GT_SWIGLU>(x, w, y, row_tiles, N, K, act, groups, x_rows, stream);
     if (epilogue == GT_STORE32) return gt_launch_grouped<GT_STORE32>(x, w, y, row_tiles, N, K, act, groups, x_rows, stream);
     if (epilogue == GT_STORE) return gt_launch_grouped<GT_STORE>(x, w, y, row_tiles, N, K, act, groups, x_rows, stream);

@@ -348,8 +348,10 @@ extern "C" int pl_moe_sort(const int* ids, const int* src, const int* fed, const
 }
 
 // out[t, :] = (1/top) sum over c of y[slot_of[t * top + c], :], the choices in their order; a pair without a slot adds nothing.
+// y may come in `splits` copies, `split_stride` floats apart, each a stretch of the product's inner width: a pair's
+// copies are added in their order.
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ slot_of,
-                                                          float* __restrict__ out, int top, int W) {
+                                                          float* __restrict__ out, int top, int W, int splits, size_t split_stride) {
     const int t = blockIdx.x;
     const float share = 1.f / static_cast<float>(top);
     for (int w = threadIdx.x * 4; w < W; w += blockDim.x * 4) {
@@ -357,7 +359,14 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
         for (int c = 0; c < top; ++c) {
             const int slot = slot_of[t * top + c];
             if (slot < 0) continue;
-            const float4 v = *reinterpret_cast<const float4*>(y + static_cast<size_t>(slot) * W + w);
+            float4 v = *reinterpret_cast<const float4*>(y + static_cast<size_t>(slot) * W + w);
+            for (int s = 1; s < splits; ++s) {
+                const float4 more = *reinterpret_cast<const float4*>(y + s * split_stride + static_cast<size_t>(slot) * W + w);
+                v.x += more.x;
+                v.y += more.y;
+                v.z += more.z;
+                v.w += more.w;
+            }
             sum.x += v.x * share;
             sum.y += v.y * share;
             sum.z += v.z * share;
@@ -367,10 +376,11 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     }
 }
 
-extern "C" int pl_moe_combine(const float* y, const int* slot_of, float* out, int n, int top, int W, hipStream_t stream) {
-    PL_REQUIRE(n >= 0 && top > 0 && W > 0 && W % 4 == 0, "moe_combine: %d rows of %d, %d a row", n, W, top);
+extern "C" int pl_moe_combine(const float* y, const int* slot_of, float* out, int n, int top, int W, int splits,
+                              long long split_stride, hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && top > 0 && W > 0 && W % 4 == 0 && splits >= 1, "moe_combine: %d rows of %d, %d a row, %d copies", n, W, top, splits);
     if (n == 0) return 0;
-    moe_combine_kernel<<<n, 256, 0, stream>>>(y, slot_of, out, top, W);
+    moe_combine_kernel<<<n, 256, 0, stream>>>(y, slot_of, out, top, W, splits, static_cast<size_t>(split_stride));
     PL_CHECK_LAUNCH("moe_combine");
     return 0;
 }

@@ -80,8 +80,8 @@ def _signatures(lib) -> None:
         "pl_softcap": [p, f, ctypes.c_long, p],
         "pl_moe_rows": [p, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, p],
         "pl_moe_sort": [p, p, p, p, p, i, i, i, i, i, i, p, p, p, p],
-        "pl_moe_combine": [p, p, p, i, i, i, p],
-        "pl_gemm_tiled_grouped": [p, p, p, p, p, ctypes.c_longlong, i, i, i, i, i, i, p],
+        "pl_moe_combine": [p, p, p, i, i, i, i, ctypes.c_longlong, p],
+        "pl_gemm_tiled_grouped": [p, p, p, p, p, ctypes.c_longlong, i, i, i, i, i, i, i, p],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name)
@@ -1564,6 +1564,16 @@ def moe_grouped_applies(x: torch.Tensor, width: int, ff: int) -> bool:
     return x.dtype == torch.bfloat16 and width % 32 == 0 and ff % 64 == 0 and _attention_mode == "kernel"
 
 
+def moe_down_splits(tiles: int, width: int, ff: int) -> int:
+    """Into how many stretches the experts' down product cuts its inner width: with few tiles of rows (decoding) its
+    launch is tiles x width / 128 workgroups that each walk the whole expert width, most of the chip idle; stretches
+    of at least 8 steps of 32 until the launch has a workgroup a compute unit."""
+    groups, splits = tiles * -(-width // 128), 1
+    while groups * splits < compute_units() and splits < 8 and ff // 32 // (splits * 2) >= 8:
+        splits *= 2
+    return splits
+
+
 def moe_grouped(x: torch.Tensor, batch, table: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
                 activation: str = "silu") -> torch.Tensor:
     """What ``moe_rows`` computes, with the step's (row, choice) pairs dealt to their experts first: an expert's
@@ -1595,9 +1605,10 @@ def moe_grouped(x: torch.Tensor, batch, table: torch.Tensor, w_gate_up: torch.Te
                            n, top, E, vocab, MOE_TILE, tiles, gather.data_ptr(), slot_of.data_ptr(), tile_group.data_ptr(), stream))
     hidden = torch.empty((slots, F), dtype=torch.bfloat16, device=x.device)
     _check(lib.pl_gemm_tiled_grouped(x.data_ptr(), w_gate_up.data_ptr(), hidden.data_ptr(), tile_group.data_ptr(),
-                                     gather.data_ptr(), 2 * F * W, tiles, n, F, W, 1, activation_code(activation), stream))
-    y = torch.empty((slots, W), dtype=torch.float32, device=x.device)
+                                     gather.data_ptr(), 2 * F * W, tiles, n, F, W, 1, activation_code(activation), 1, stream))
+    splits = moe_down_splits(tiles, W, F)
+    y = torch.empty((splits, slots, W), dtype=torch.float32, device=x.device)
     _check(lib.pl_gemm_tiled_grouped(hidden.data_ptr(), w_down.data_ptr(), y.data_ptr(), tile_group.data_ptr(), 0,
-                                     W * F, tiles, slots, W, F, 3, 0, stream))
-    _check(lib.pl_moe_combine(y.data_ptr(), slot_of.data_ptr(), out.data_ptr(), n, top, W, stream))
+                                     W * F, tiles, slots, W, F, 3, 0, splits, stream))
+    _check(lib.pl_moe_combine(y.data_ptr(), slot_of.data_ptr(), out.data_ptr(), n, top, W, splits, slots * W, stream))
     return out
