@@ -30,8 +30,10 @@ struct HcArgs {
     int S, W;
 };
 
-template <typename T>
-__global__ __launch_bounds__(256) void hc_step_kernel(HcArgs a) {
+// VEC: how many neighbouring columns a thread takes at a time (4: every load and store is 16 bytes, and a row of
+// up to 4,096 values is one round of loads for a workgroup of 1,024 threads, all of them asked for at once).
+template <typename T, int VEC>
+__global__ __launch_bounds__(1024) void hc_step_kernel(HcArgs a) {
     extern __shared__ float hc_row[];                 // the read-out's row before its norm, then 16 floats of scratch
     float* scratch = hc_row + a.W;
     const int i = blockIdx.x;
@@ -52,48 +54,66 @@ __global__ __launch_bounds__(256) void hc_step_kernel(HcArgs a) {
 #pragma unroll
         for (int s = 0; s < HC_MAX_COPIES; ++s) in[s] = s < S ? a.in[s] : 0.f;
     }
+    typedef float vec_t __attribute__((ext_vector_type(VEC)));
     float ss = 0.f;
-    for (int c = threadIdx.x; c < W; c += blockDim.x) {
-        float v[HC_MAX_COPIES];
+    for (int c = threadIdx.x * VEC; c < W; c += blockDim.x * VEC) {
+        vec_t v[HC_MAX_COPIES];
 #pragma unroll
-        for (int s = 0; s < HC_MAX_COPIES; ++s) v[s] = s < S ? x[static_cast<size_t>(s) * W + c] : 0.f;
+        for (int s = 0; s < HC_MAX_COPIES; ++s) {
+            if (s < S) v[s] = *reinterpret_cast<const vec_t*>(x + static_cast<size_t>(s) * W + c);
+            else v[s] = vec_t(0.f);
+        }
         if (y != nullptr) {
-            const float add = y[c];
-            float nv[HC_MAX_COPIES];
+            const vec_t add = *reinterpret_cast<const vec_t*>(y + c);
+            vec_t nv[HC_MAX_COPIES];
 #pragma unroll
             for (int t = 0; t < HC_MAX_COPIES; ++t) {
-                float acc = 0.f;
+                vec_t acc = vec_t(0.f);
 #pragma unroll
                 for (int s = 0; s < HC_MAX_COPIES; ++s)
-                    if (s < S) acc = fmaf(mix[s * HC_MAX_COPIES + t], v[s], acc);
-                nv[t] = fmaf(out[t], add, acc);
+                    if (s < S) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) acc[e] = fmaf(mix[s * HC_MAX_COPIES + t], v[s][e], acc[e]);
+                    }
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) nv[t][e] = fmaf(out[t], add[e], acc[e]);
             }
 #pragma unroll
             for (int t = 0; t < HC_MAX_COPIES; ++t) {
                 v[t] = nv[t];
-                if (t < S) x[static_cast<size_t>(t) * W + c] = nv[t];
+                if (t < S) *reinterpret_cast<vec_t*>(x + static_cast<size_t>(t) * W + c) = nv[t];
             }
         }
         if (a.in != nullptr) {
-            float u = 0.f;
+            vec_t u = vec_t(0.f);
 #pragma unroll
             for (int s = 0; s < HC_MAX_COPIES; ++s)
-                if (s < S) u = fmaf(in[s], v[s], u);
-            hc_row[c] = u;
-            ss += u * u;
+                if (s < S) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) u[e] = fmaf(in[s], v[s][e], u[e]);
+                }
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                hc_row[c + e] = u[e];
+                ss += u[e] * u[e];
+            }
         }
     }
     if (a.in == nullptr) return;
     T* o = static_cast<T*>(a.read) + static_cast<size_t>(i) * W;
     if (a.gain == nullptr) {
         // (every thread reads back what it wrote itself)
-        for (int c = threadIdx.x; c < W; c += blockDim.x) o[c] = from_float<T>(hc_row[c]);
+        for (int c = threadIdx.x * VEC; c < W; c += blockDim.x * VEC)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o[c + e] = from_float<T>(hc_row[c + e]);
         return;
     }
     ss = block_sum(ss, scratch);
     const float inv = 1.f / sqrtf(ss / static_cast<float>(W) + a.eps);
     const float* gain = static_cast<const float*>(a.gain);
-    for (int c = threadIdx.x; c < W; c += blockDim.x) o[c] = from_float<T>(hc_row[c] * inv * gain[c]);
+    for (int c = threadIdx.x * VEC; c < W; c += blockDim.x * VEC)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o[c + e] = from_float<T>(hc_row[c + e] * inv * gain[c + e]);
 }
 
 // streams [n, S, W] (32-bit) in place.  y, mix, out: the rebuild behind a sublayer (all null: none).  in: the
@@ -111,10 +131,18 @@ extern "C" int pl_hc_step(float* streams, const float* y, const float* mix, cons
     if (count == 0 || (y == nullptr && in == nullptr)) return 0;
     HcArgs a{streams, y, mix, out, in, gain, eps, read, rows, S, W};
     const size_t lds = (static_cast<size_t>(W) + 16) * sizeof(float);
-    const int threads = W >= 1024 ? 256 : (W >= 256 ? 128 : 64);
-    if (dtype == PL_DTYPE_F32) hc_step_kernel<float><<<count, threads, lds, stream>>>(a);
-    else if (dtype == PL_DTYPE_BF16) hc_step_kernel<bf16_t><<<count, threads, lds, stream>>>(a);
-    else PL_REQUIRE(false, "hc_step: dtype code %d", dtype);
+    PL_REQUIRE(dtype == PL_DTYPE_F32 || dtype == PL_DTYPE_BF16, "hc_step: dtype code %d", dtype);
+    if (W % 4 == 0) {
+        // a thread a quad of columns, one round of loads up to a width of 4,096
+        int threads = ((W / 4 + 63) / 64) * 64;
+        threads = threads > 1024 ? 1024 : threads;
+        if (dtype == PL_DTYPE_F32) hc_step_kernel<float, 4><<<count, threads, lds, stream>>>(a);
+        else hc_step_kernel<bf16_t, 4><<<count, threads, lds, stream>>>(a);
+    } else {
+        const int threads = W >= 1024 ? 256 : (W >= 256 ? 128 : 64);
+        if (dtype == PL_DTYPE_F32) hc_step_kernel<float, 1><<<count, threads, lds, stream>>>(a);
+        else hc_step_kernel<bf16_t, 1><<<count, threads, lds, stream>>>(a);
+    }
     PL_CHECK_LAUNCH("hc_step");
     return 0;
 }
