@@ -41,18 +41,31 @@ __global__ __launch_bounds__(1024) void hc_step_kernel(HcArgs a) {
     const int S = a.S, W = a.W;
     float* x = a.streams + static_cast<size_t>(r) * S * W;
     const float* y = a.y != nullptr ? a.y + static_cast<size_t>(r) * W : nullptr;
-    float mix[HC_MAX_COPIES * HC_MAX_COPIES], out[HC_MAX_COPIES], in[HC_MAX_COPIES];
-    if (y != nullptr) {
-#pragma unroll
-        for (int s = 0; s < HC_MAX_COPIES; ++s) {
-            out[s] = s < S ? a.out[s] : 0.f;
-#pragma unroll
-            for (int t = 0; t < HC_MAX_COPIES; ++t) mix[s * HC_MAX_COPIES + t] = (s < S && t < S) ? a.mix[s * S + t] : 0.f;
+    // The weights travel through LDS: the first eighty threads ask for one of them each, all at once
+    // (read one after the other from where they lie, each behind a condition, they were eighty trips to memory in a row).
+    __shared__ float hc_w[HC_MAX_COPIES * HC_MAX_COPIES + 2 * HC_MAX_COPIES];
+    for (int k = threadIdx.x; k < HC_MAX_COPIES * HC_MAX_COPIES + 2 * HC_MAX_COPIES; k += blockDim.x) {
+        if (k < HC_MAX_COPIES * HC_MAX_COPIES) {
+            const int s = k / HC_MAX_COPIES, t = k % HC_MAX_COPIES;
+            hc_w[k] = (y != nullptr && s < S && t < S) ? a.mix[s * S + t] : 0.f;
+        } else if (k < HC_MAX_COPIES * HC_MAX_COPIES + HC_MAX_COPIES) {
+            const int t = k - HC_MAX_COPIES * HC_MAX_COPIES;
+            hc_w[k] = (y != nullptr && t < S) ? a.out[t] : 0.f;
+        } else if (k < HC_MAX_COPIES * HC_MAX_COPIES + 2 * HC_MAX_COPIES) {
+            const int t = k - HC_MAX_COPIES * HC_MAX_COPIES - HC_MAX_COPIES;
+            hc_w[k] = (a.in != nullptr && t < S) ? a.in[t] : 0.f;
         }
     }
-    if (a.in != nullptr) {
+    __syncthreads();
+    // (the same for every lane: kept in scalar registers)
+    auto uniform = [&](int k) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(hc_w[k]))); };
+    float mix[HC_MAX_COPIES * HC_MAX_COPIES], out[HC_MAX_COPIES], in[HC_MAX_COPIES];
 #pragma unroll
-        for (int s = 0; s < HC_MAX_COPIES; ++s) in[s] = s < S ? a.in[s] : 0.f;
+    for (int k = 0; k < HC_MAX_COPIES * HC_MAX_COPIES; ++k) mix[k] = uniform(k);
+#pragma unroll
+    for (int k = 0; k < HC_MAX_COPIES; ++k) {
+        out[k] = uniform(HC_MAX_COPIES * HC_MAX_COPIES + k);
+        in[k] = uniform(HC_MAX_COPIES * HC_MAX_COPIES + HC_MAX_COPIES + k);
     }
     typedef float vec_t __attribute__((ext_vector_type(VEC)));
     float ss = 0.f;
