@@ -1561,7 +1561,7 @@ MOE_TILE = 128       # rows of a tile of the grouped product
 def moe_grouped_applies(x: torch.Tensor, width: int, ff: int) -> bool:
     """Whether the experts of a step run as grouped products on the matrix cores: bfloat16, an inner width the
     tiles take (a multiple of 32), an expert width that is a multiple of 64."""
-    return x.dtype == torch.bfloat16 and width % 32 == 0 and ff % 64 == 0 and _attention_mode == "kernel"
+    return x.dtype == torch.bfloat16 and width % 32 == 0 and ff % 64 == 0
 
 
 def moe_down_splits(tiles: int, width: int, ff: int) -> int:

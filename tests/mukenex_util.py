@@ -191,12 +191,12 @@ def drawn_config(seed: int) -> dict:
             rank, rot = rng.choice([16, 32, 48, 64, 96, 112, 160, 192, 224]), rng.choice([2, 8, 16, 32, 64])
             turned = rot if rng.random() < 0.8 else max(2, rot // 2 // 2 * 2)
             layers.append(latent(heads, dim, rot, vdim, rank, (dim + rot) ** -0.5, base=rng.choice([100.0, 10000.0, 250000.0]),
-                                 turned=turned, window=rng.choice([None, 3, 20, 64, 72, 100, 500]), mlp=feed_forward()))
+                                 turned=turned, window=rng.choice([None, 3, 20, 64, 70, 100, 500]), mlp=feed_forward()))
         elif kind < 0.7:
             kv_heads, group = rng.choice([1, 2, 4]), rng.choice([1, 2, 4, 8])
             dim, vdim = rng.choice([16, 32, 48, 64, 96, 128]), rng.choice([16, 32, 48, 64, 96, 128])
             layers.append(attention(kv_heads * group, kv_heads, dim, vdim, rng.choice([0.5, 1.0, 2.0]) * dim ** -0.5,
-                                    block=rng.choice([None, 3, 20, 64, 72, 100, 500]), mlp=feed_forward()))
+                                    block=rng.choice([None, 3, 20, 48, 70, 100, 500]), mlp=feed_forward()))
         else:
             heads = rng.choice([1, 2, 4, 6])
             layers.append(lightning(heads, rng.choice([8, 16, 32, 64]), rng.choice([8, 16, 32, 64]),
