@@ -1,6 +1,7 @@
 // What attention layers without a gain on q and k do between their projections and the attention kernels.
 //
-// head_prepare: for every token and head of a projected row [q | k | v] (32-bit sums): q and k divided by
+// head_prepare: for every token and head of a projected row [q | k | v] (32-bit sums, plus the projections' biases
+// where they have any): q and k divided by
 // their root mean square over the head (optional, with an optional gain), the rotation of a stretch of the
 // head (optional: value 2i with value 2i + 1, from tables of cosines and sines), q times a temperature that
 // grows with the logarithm of the position (optional), then q into the query buffer and k and v into the
@@ -18,6 +19,7 @@
 
 struct HeadPrepareArgs {
     const float* rows;        // [n, stride]: q | k | v from column `off`
+    const float* bias;        // [H D + G D + G V] added to q | k | v first, or null
     int stride, off;
     int unit;                 // q and k divided by their root mean square
     float eps;
@@ -53,10 +55,11 @@ __global__ __launch_bounds__(64) void head_prepare_kernel(HeadPrepareArgs a) {
     const int width = kind == 2 ? V : D;
     const int c0 = kind == 0 ? index * D : (kind == 1 ? H * D + index * D : H * D + G * D + index * V);
     const float* src = a.rows + static_cast<size_t>(t) * a.stride + a.off + c0;
+    const float* bias = a.bias != nullptr ? a.bias + c0 : nullptr;
 
     float ss = 0.f;
     for (int e = lane; e < width; e += 64) {
-        const float x = src[e];
+        const float x = bias != nullptr ? src[e] + bias[e] : src[e];
         head[e] = x;
         ss += x * x;
     }
@@ -102,7 +105,7 @@ __global__ __launch_bounds__(64) void head_prepare_kernel(HeadPrepareArgs a) {
     }
 }
 
-extern "C" int pl_head_prepare(const float* rows, int stride, int off, int unit, float eps, const float* q_gain,
+extern "C" int pl_head_prepare(const float* rows, const float* bias, int stride, int off, int unit, float eps, const float* q_gain,
                                const float* k_gain, const float* cos, const float* sin, int rot_off, int rot,
                                int table_rows, int tempered, float temp_coef, int temp_every, const int* positions,
                                const int* seq_of, const int* block_table, int max_blocks, int block_size, int write_kv,
@@ -115,7 +118,7 @@ extern "C" int pl_head_prepare(const float* rows, int stride, int off, int unit,
     PL_REQUIRE(block_size > 0 && max_blocks > 0 && (!tempered || temp_every > 0), "head_prepare: pages of %d, tables of %d, a temperature every %d", block_size, max_blocks, temp_every);
     PL_REQUIRE(stride >= off + H * D + G * D + G * V, "head_prepare: rows of %d values for %d + %d + %d from %d on", stride, H * D, G * D, G * V, off);
     if (n == 0) return 0;
-    HeadPrepareArgs a{rows, stride, off, unit, eps, q_gain, k_gain, cos, sin, rot_off, rot, table_rows, tempered, temp_coef,
+    HeadPrepareArgs a{rows, bias, stride, off, unit, eps, q_gain, k_gain, cos, sin, rot_off, rot, table_rows, tempered, temp_coef,
                       temp_every, positions, seq_of, block_table, max_blocks, block_size, write_kv, q_out, k_pool, v_pool,
                       H, G, D, V, Dp};
     const dim3 grid(n, H + 2 * G);

@@ -349,6 +349,7 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* ids, const in
     };
     for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
         const int e = expert_of(p);
+        slot_of[p] = e;                               // (kept for the second pass, which the same thread makes)
         if (e >= 0) atomicAdd(&count[e], 1);
     }
     __syncthreads();
@@ -364,7 +365,7 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* ids, const in
     }
     __syncthreads();
     for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
-        const int e = expert_of(p);
+        const int e = slot_of[p];
         int slot = -1;
         if (e >= 0) {
             slot = base[e] + atomicAdd(&cursor[e], 1);

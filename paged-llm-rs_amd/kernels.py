@@ -37,7 +37,7 @@ def _signatures(lib) -> None:
         "pl_gemm_plain": [p, p, p, i, i, i, i, i, i, i, p],
         "pl_paged_attention_plain": [p, i, p, p, p, p, i, i, p, p, i, i, i, i, f, i, i, p, p, p],
         "pl_gemm_heads": [p, p, p, i, i, i, i, i, ctypes.c_long, i, ctypes.c_long, i, i, p],
-        "pl_head_prepare": [p, i, i, i, f, p, p, p, p, i, i, i, i, f, i, p, p, p, i, i, i, p, p, p, i, i, i, i, i, i, i, p],
+        "pl_head_prepare": [p, p, i, i, i, f, p, p, p, p, i, i, i, i, f, i, p, p, p, i, i, i, p, p, p, i, i, i, i, i, i, i, p],
         "pl_latent_prepare": [p, i, i, i, p, f, p, p, i, i, p, p, p, i, i, i, p, p, p, i, i, i, i, i, i, i, p],
         "pl_head_gate": [p, i, p, i, i, p, i, i, i, i, p],
         "pl_add_position_rows": [p, p, i, p, i, i, i, p],
@@ -1367,12 +1367,14 @@ GEMM_HEADS_PLAIN_ROWS = 0
 
 def head_prepare(rows: torch.Tensor, off: int, batch, kv, q_out: torch.Tensor, H: int, G: int, D: int, V: int,
                  padded: int, unit_eps: float | None = None, q_gain=None, k_gain=None, cos=None, sin=None,
-                 rot_off: int = 0, rot: int = 0, temperature: tuple | None = None, write_kv: bool = True) -> None:
+                 rot_off: int = 0, rot: int = 0, temperature: tuple | None = None, write_kv: bool = True,
+                 bias: torch.Tensor | None = None) -> None:
     """Between an attention layer's projections and the attention kernels: ``rows`` [n, >= off + H D + G D + G V]
     (32-bit) holds q | k | v from column ``off``.  q and k are divided by their root mean square over a head
     (``unit_eps``; times a gain where one is given), ``rot`` values from ``rot_off`` on turn in pairs (2i, 2i + 1)
     by the tables' angles, q is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1) (``temperature`` =
-    (coef, every)); q goes to ``q_out`` [n, H * padded], k and v into the pages, every head in ``padded`` values."""
+    (coef, every)); q goes to ``q_out`` [n, H * padded], k and v into the pages, every head in ``padded`` values.
+    ``bias`` (32-bit, [H D + G D + G V]): the projections' biases, added to q | k | v before anything else."""
     n = rows.shape[0]
     _need(rows, "projected rows", None, torch.float32)
     if rows.dim() != 2:
@@ -1393,8 +1395,10 @@ def head_prepare(rows: torch.Tensor, off: int, batch, kv, q_out: torch.Tensor, H
             raise TensorError(f"rotary tables have shape {tuple(cos.shape)}, expected [positions, {rot // 2}]")
         table_rows = cos.shape[0]
     coef, every = temperature if temperature is not None else (0.0, 1)
+    if bias is not None:
+        _need(bias, "biases of q, k and v", (H * D + G * D + G * V,), torch.float32)
     _check(library().pl_head_prepare(
-        rows.data_ptr(), rows.shape[1], int(off), 1 if unit_eps is not None else 0, float(unit_eps or 0.0),
+        rows.data_ptr(), _ptr(bias), rows.shape[1], int(off), 1 if unit_eps is not None else 0, float(unit_eps or 0.0),
         _ptr(q_gain), _ptr(k_gain), _ptr(cos) if rot else 0, _ptr(sin) if rot else 0, int(rot_off), int(rot), table_rows,
         1 if temperature is not None else 0, float(coef), int(every), batch.positions.data_ptr(),
         batch.seq_of.data_ptr(), kv.block_table.data_ptr(), kv.block_table.shape[1], kv.block_size,

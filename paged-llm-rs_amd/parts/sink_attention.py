@@ -87,8 +87,11 @@ class SinkAttention:
         self.window = int(spec.window or 0)
         # what the attention kernels are told: a window as it is, blocks of positions as a negative number
         self.mask = -self.window if spec.mask == "block" else self.window
-        biases = [params["q.b"], params["k.b"], params["v.b"]] if spec.qkv_bias else None
-        self.proj = Linear.fused([params["q"], params["k"], params["v"]], biases)
+        # (the biases are added where the projection's 32-bit sums are read next, in the prepare kernel: the product
+        # keeps what it fuses, and a pass over the rows is saved)
+        self.bias = (torch.cat([params["q.b"], params["k.b"], params["v.b"]]).to(torch.float32).contiguous()
+                     if spec.qkv_bias else None)
+        self.proj = Linear.fused([params["q"], params["k"], params["v"]])
         self.q_gain = params["q.norm"].to(torch.float32).contiguous() if spec.qk_gain else None
         self.k_gain = params["k.norm"].to(torch.float32).contiguous() if spec.qk_gain else None
         self.sinks = head_sinks(spec.sink, H, params, device)
@@ -118,7 +121,7 @@ class SinkAttention:
         q = torch.empty((n, self.H * self.padded), dtype=self.dtype, device=rows.device)
         kernels.head_prepare(rows, 0, batch, kv, q, self.H, self.G, self.D, self.V, self.padded,
                              unit_eps=self.spec.qk_unit_eps, q_gain=self.q_gain, k_gain=self.k_gain,
-                             temperature=self.temperature, write_kv=ctx.writes_cache)
+                             temperature=self.temperature, write_kv=ctx.writes_cache, bias=self.bias)
         out = torch.empty((n, self.H * self.padded), dtype=self.dtype, device=rows.device)
         kernels.sink_attention(q, out, batch, kv, self.H, self.G, self.padded, self.scale, self.mask,
                                sinks=self.sinks, slopes=self.slopes)
