@@ -341,6 +341,49 @@ __global__ __launch_bounds__(64) void gated_group_norm_kernel(const float* __res
     }
 }
 
+// The same for groups of more than 512 columns (all heads normalised together): a workgroup of four waves a row and
+// group, so that a group of up to 2,048 is read once, every load asked for at once.
+template <typename T>
+__global__ __launch_bounds__(256) void gated_group_norm_wide_kernel(const float* __restrict__ x, int width, int group,
+                                                                    const float* __restrict__ gain, int gain_len, float eps,
+                                                                    const float* __restrict__ gate, int gate_stride,
+                                                                    int gate_off, int act, T* __restrict__ out) {
+    __shared__ float scratch[16];
+    const int t = blockIdx.x, first = blockIdx.y * group;
+    const float* row = x + static_cast<size_t>(t) * width + first;
+    const float* g = gate != nullptr ? gate + static_cast<size_t>(t) * gate_stride + gate_off + first : nullptr;
+    const float* gains = gain + (gain_len == width ? first : 0);     // (gain_len is the row's width or the group's)
+    constexpr int KEEP = 8;
+    float kept[KEEP], gates[KEEP], scale[KEEP];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+        const int e = threadIdx.x + 256 * k;
+        kept[k] = e < group ? row[e] : 0.f;
+        gates[k] = (e < group && act >= 0) ? g[e] : 0.f;
+        scale[k] = e < group ? gains[e] : 0.f;
+        ss += kept[k] * kept[k];
+    }
+    for (int e = threadIdx.x + 256 * KEEP; e < group; e += 256) ss += row[e] * row[e];
+    ss = block_sum(ss, scratch);
+    const float inv = 1.f / sqrtf(ss / static_cast<float>(group) + eps);
+    T* o = out + static_cast<size_t>(t) * width + first;
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+        const int e = threadIdx.x + 256 * k;
+        if (e < group) {
+            float y = kept[k] * inv * scale[k];
+            if (act >= 0) y *= act == 0 ? sigmoid_f(gates[k]) : silu_f(gates[k]);
+            o[e] = from_float<T>(y);
+        }
+    }
+    for (int e = threadIdx.x + 256 * KEEP; e < group; e += 256) {
+        float y = row[e] * inv * gains[e];
+        if (act >= 0) y *= act == 0 ? sigmoid_f(g[e]) : silu_f(g[e]);
+        o[e] = from_float<T>(y);
+    }
+}
+
 extern "C" int pl_gated_group_norm(const float* x, int n, int width, int group, const float* gain, int gain_len,
                                    float eps, const float* gate, int gate_stride, int gate_off, int act, void* out,
                                    int dtype, hipStream_t stream) {
@@ -351,6 +394,14 @@ extern "C" int pl_gated_group_norm(const float* x, int n, int width, int group, 
     if (n == 0) return 0;
     PL_REQUIRE(width / group <= 65535, "gated_group_norm: %d groups a row", width / group);
     const dim3 grid(n, width / group);
+    if (group > 512 && (dtype == PL_DTYPE_F32 || dtype == PL_DTYPE_BF16)) {
+        if (dtype == PL_DTYPE_F32)
+            gated_group_norm_wide_kernel<float><<<grid, 256, 0, stream>>>(x, width, group, gain, gain_len, eps, gate, gate_stride, gate_off, act, static_cast<float*>(out));
+        else
+            gated_group_norm_wide_kernel<bf16_t><<<grid, 256, 0, stream>>>(x, width, group, gain, gain_len, eps, gate, gate_stride, gate_off, act, static_cast<bf16_t*>(out));
+        PL_CHECK_LAUNCH("gated_group_norm");
+        return 0;
+    }
     if (dtype == PL_DTYPE_F32)
         gated_group_norm_kernel<float><<<grid, 64, 0, stream>>>(x, width, group, gain, gain_len, eps, gate, gate_stride, gate_off, act, static_cast<float*>(out));
     else if (dtype == PL_DTYPE_BF16)

@@ -131,6 +131,32 @@ def test_the_pass_over_the_copies_of_the_stream(copies, width):
     assert torch.equal(wide.view(n, copies, width), dev(y)[:, None, :].expand(n, copies, width))
 
 
+@pytest.mark.parametrize("width,group,gains", [(120, 120, 120), (1024, 1024, 1024), (2048, 1024, 2048), (2560, 2560, 2560),
+                                                (640, 640, 640), (3000, 1500, 1500), (1024, 128, 128)])
+@pytest.mark.parametrize("act", [None, "sigmoid", "silu"])
+def test_the_norm_over_all_heads_of_a_state_layers_read_out(width, group, gains, act):
+    """Groups of a head up to the whole row (above 512 columns a workgroup of four waves takes a group, above 2,048 in two
+    rounds), a gain a column of the row or of a group, no gate and both kinds, against 64-bit arithmetic."""
+    from paged_llm_rs_amd import kernels
+
+    g = torch.Generator().manual_seed(width + group)
+    n, off = 19, 5
+    x = torch.randn((n, width), generator=g, dtype=torch.float64) * 2
+    gain = 1 + 0.3 * torch.randn((gains,), generator=g, dtype=torch.float64)
+    gate = torch.randn((n, off + width + 3), generator=g, dtype=torch.float64)
+    eps = 1e-5
+    grouped = x.view(n, width // group, group)
+    want = (grouped / torch.sqrt((grouped * grouped).mean(-1, keepdim=True) + eps)).reshape(n, width)
+    want = want * (gain if gains == width else gain.repeat(width // group))
+    if act is not None:
+        chosen = gate[:, off:off + width]
+        want = want * (torch.sigmoid(chosen) if act == "sigmoid" else chosen * torch.sigmoid(chosen))
+    for dtype, tol in ((torch.float32, 3e-6), (torch.bfloat16, 8e-3)):
+        got = kernels.gated_group_norm(x.float().cuda(), group, gain.float().cuda(), eps, dtype,
+                                       gate=gate.float().cuda() if act else None, gate_off=off if act else 0, gate_act=act)
+        assert got.dtype == dtype and (got.double().cpu() - want).abs().max() <= tol * want.abs().max()
+
+
 class _Rows:
     """What the experts' kernels read of a step."""
 
