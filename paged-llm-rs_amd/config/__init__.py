@@ -1,3 +1,4 @@
+from .dimalix import DimalixConfig
 from .generation import GenerationConfig
 from .lefavik import LefavikConfig
 from .mukenex import MukenexConfig
@@ -8,7 +9,7 @@ from .specs import (AttentionSpec, GatedMlpSpec, LayerSpec, ModelSpec, NormSpec,
                     ScheduleEntry)
 
 __all__ = [
-    "GenerationConfig", "Qwen3Config", "PapivikConfig", "LefavikConfig", "MukenexConfig", "read_json", "architectures", "config_class_for",
+    "GenerationConfig", "Qwen3Config", "PapivikConfig", "LefavikConfig", "MukenexConfig", "DimalixConfig", "read_json", "architectures", "config_class_for",
     "load_config", "register_architecture", "AttentionSpec", "GatedMlpSpec", "LayerSpec",
     "ModelSpec", "NormSpec", "PositionSpec", "ScheduleEntry",
 ]

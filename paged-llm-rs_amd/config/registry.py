@@ -9,6 +9,7 @@ from __future__ import annotations
 from pathlib import Path
 
 from ..errors import ConfigError, UnsupportedError
+from .dimalix import DimalixConfig
 from .lefavik import LefavikConfig
 from .mukenex import MukenexConfig
 from .papivik import PapivikConfig
@@ -68,3 +69,4 @@ register_architecture("Qwen3ForCausalLM", Qwen3Config, model_type="qwen3")
 register_architecture("Papivik", PapivikConfig, model_type="papivik")
 register_architecture("Lefavik", LefavikConfig, model_type="lefavik")
 register_architecture("Mukenex", MukenexConfig, model_type="mukenex")
+register_architecture("Dimalix", DimalixConfig, model_type="dimalix")

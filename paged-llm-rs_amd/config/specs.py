@@ -65,6 +65,7 @@ class LayerSpec:
     weight_prefix: str = ""
     names: Optional[dict] = None            # other tensor-name parts for the block's members (norm1, mixer, norm2, feed_forward)
     stream_copies: Optional[int] = None     # for an arrangement over several copies of the stream: how many
+    layer_scale: bool = False               # a sublayer's output times a gain a column before it joins the stream (``ls1``, ``ls2``)
 
 
 @dataclass(frozen=True)
@@ -78,6 +79,9 @@ class ScheduleEntry:
     # runs with different ``cache_key`` (any numbers; None is the layer's own index) share nothing.  ``cache_from``
     # names the key that is read.
     cache_key: Optional[int] = None
+    # The stream as it was right behind the embedding (and its transforms) is added to the stream before this run:
+    # a stretch of layers that runs again starts every further pass from what it left plus what the model began with.
+    add_embedding: bool = False
 
 
 @dataclass(frozen=True)
@@ -225,6 +229,8 @@ class LatentAttentionSpec:
     gate_each: str = "head"                 # one gate a "head" (tensor ``g`` [heads, width]) or an "element" ([heads * value_dim, width])
     window: Optional[int] = None
     borrows: bool = False                   # no projection onto the small vector: the schedule names the layer whose pages are read
+    # the rotation's frequencies rescaled by wavelength: (factor, low, high, original), see ``TiedAttentionSpec``
+    rotary_scaling: Optional[tuple] = None
 
 
 # ---- several copies of the stream, experts chosen by a table ----------------------------------------
@@ -239,3 +245,51 @@ class TableExpertsSpec:
     intermediate_size: int = 0
     vocab_size: int = 0
     activation: str = "silu"
+
+
+# ---- values that are the keys, a norm over all heads at once, experts behind a router ------------------
+
+@dataclass(frozen=True)
+class TiedAttentionSpec:
+    """Grouped-query softmax attention over a paged cache without a value projection: a token's values are its keys
+    as projected (bias included), before the keys are normed and turned.  q and k may carry biases; ``qk_norm_eps``
+    norms q over ALL its heads at once (one root mean square over the whole projection, a gain a column, tensors
+    ``q.norm`` and ``k.norm``) and k likewise; the first ``rotary_dims`` values of every head turn in pairs
+    (2i, 2i + 1) by position * f_i, f_i = base^(-2i/dims).  ``rotary_scaling`` = (factor, low, high, original)
+    rescales the frequencies by their wavelength l = 2 pi / f: kept where l < original / high, divided by factor
+    where l > original / low, and between the two blended by s = (original / l - low) / (high - low)."""
+    kind: str = "tied_attention"
+    num_heads: int = 0
+    num_kv_heads: int = 0
+    head_dim: int = 0
+    scale: Optional[float] = None           # None = 1/sqrt(head_dim)
+    qk_bias: bool = False                   # tensors ``q.b`` and ``k.b``
+    qk_norm_eps: Optional[float] = None     # None: q and k are used as projected
+    rotary_dims: int = 0                    # 0: no rotation
+    rotary_base: float = 10000.0
+    rotary_scaling: Optional[tuple] = None
+    window: Optional[int] = None            # the size of the window or of the blocks; None: every key up to the query
+    mask: str = "window"                    # "window" or "block", as in SinkAttentionSpec
+
+
+@dataclass(frozen=True)
+class RoutedExpertsSpec:
+    """``experts`` small gated feed-forwards, down(act(gate x) * (up x)), and behind them ``identity`` experts whose
+    output is their input, of which a token uses the ``top`` that a router chooses.  The router's logits (tensor
+    ``router`` [experts + identity, width], 32-bit sums) pass ``score`` (softmax over all of them); the choice is by
+    score plus ``correction`` (a tensor of that name, where ``corrected``); experts form ``groups`` equal groups of
+    neighbours, a group counts by its best choice score, and only experts of the best ``groups_kept`` groups can be
+    chosen (``groups`` 1: no groups).  A chosen expert weighs its score (without the correction), divided, where
+    ``normalised``, by the chosen scores' sum plus ``weight_eps``."""
+    kind: str = "routed_experts"
+    experts: int = 0
+    identity: int = 0
+    top: int = 0
+    intermediate_size: int = 0
+    activation: str = "silu"
+    score: str = "softmax"
+    corrected: bool = True
+    groups: int = 1
+    groups_kept: int = 1
+    normalised: bool = True
+    weight_eps: float = 1e-20

@@ -129,6 +129,124 @@ extern "C" int pl_head_prepare(const float* rows, const float* bias, int stride,
     return 0;
 }
 
+// ---- q and k normed over all their heads at once, values that are the keys as projected ------------------------
+
+struct WidePrepareArgs {
+    const float* rows;        // [n, stride]: q | k from column `off`
+    const float* bias;        // [H D + G D] added to q | k first, or null
+    int stride, off;
+    int normed;               // q divided by its root mean square over all H D values, k over all G D
+    float eps;
+    const float* q_gain;      // [H D] or null
+    const float* k_gain;      // [G D] or null
+    const float* freq;        // [rot / 2]: the angle of pair i is position * freq[i], in 32-bit
+    int rot;                  // the first `rot` values of every head turn in pairs (2i, 2i + 1)
+    const int* positions;
+    const int* seq_of;
+    const int* block_table;
+    int max_blocks, block_size, write_kv;
+    void* q_out;              // [n, H * Dp]
+    void* k_pool;             // [pages * block_size, G * Dp]: the keys, normed and turned
+    void* v_pool;             // the same shape: the keys as projected (bias included)
+    int H, G, D, Dp;
+};
+
+// A workgroup a token.  The row of q | k (with the biases) waits in LDS; two sums of squares over the whole
+// projections; then every value is normed, gained, turned and stored, heads in rows of Dp values with zeros behind.
+template <typename T>
+__global__ __launch_bounds__(256) void wide_prepare_kernel(WidePrepareArgs a) {
+    extern __shared__ float wide_lds[];               // [H D + G D] values, [rot / 2] cosines, [rot / 2] sines
+    __shared__ float scratch[16];
+    const int t = blockIdx.x;
+    const int pos = a.positions[t];
+    if (pos < 0) return;
+    const int H = a.H, G = a.G, D = a.D, Dp = a.Dp, half = a.rot / 2;
+    const int nq = H * D, nk = a.write_kv ? G * D : 0;
+    float* vals = wide_lds;
+    float* cs = wide_lds + H * D + G * D;
+    float* sn = cs + half;
+    const float* src = a.rows + static_cast<size_t>(t) * a.stride + a.off;
+    float ssq = 0.f, ssk = 0.f;
+    for (int e = threadIdx.x; e < nq + nk; e += blockDim.x) {
+        const float x = a.bias != nullptr ? src[e] + a.bias[e] : src[e];
+        vals[e] = x;
+        if (e < nq) ssq += x * x;
+        else ssk += x * x;
+    }
+    for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(static_cast<float>(pos) * a.freq[i], &sn[i], &cs[i]);
+    float inv_q = 1.f, inv_k = 1.f;
+    if (a.normed) {
+        ssq = block_sum(ssq, scratch);
+        inv_q = 1.f / sqrtf(ssq / static_cast<float>(nq) + a.eps);
+        if (nk > 0) {
+            ssk = block_sum(ssk, scratch);
+            inv_k = 1.f / sqrtf(ssk / static_cast<float>(nk) + a.eps);
+        }
+    }
+    __syncthreads();
+    T* q_dst = static_cast<T*>(a.q_out) + static_cast<size_t>(t) * H * Dp;
+    T* k_dst = nullptr;
+    T* v_dst = nullptr;
+    if (nk > 0) {
+        const int s = a.seq_of[t];
+        const int page = a.block_table[static_cast<size_t>(s) * a.max_blocks + pos / a.block_size];
+        if (page >= 0) {
+            const size_t row = static_cast<size_t>(page) * a.block_size + pos % a.block_size;
+            k_dst = static_cast<T*>(a.k_pool) + row * G * Dp;
+            v_dst = static_cast<T*>(a.v_pool) + row * G * Dp;
+        }
+    }
+    const int total = (H + (k_dst != nullptr ? G : 0)) * Dp;
+    for (int e = threadIdx.x; e < total; e += blockDim.x) {
+        const int head = e / Dp, d = e - head * Dp;
+        const bool query = head < H;
+        const int c = query ? head * D + d : nq + (head - H) * D + d;      // the value's place in `vals`
+        float x = 0.f, raw = 0.f;
+        if (d < D) {
+            const float inv = query ? inv_q : inv_k;
+            const float* gain = query ? a.q_gain : a.k_gain;
+            const int g0 = query ? 0 : nq;
+            raw = vals[c];
+            x = raw * inv * (gain != nullptr ? gain[c - g0] : 1.f);
+            if (d < a.rot) {
+                const int other = (d & 1) ? c - 1 : c + 1;
+                const float y = vals[other] * inv * (gain != nullptr ? gain[other - g0] : 1.f);
+                const int i = d >> 1;
+                x = (d & 1) ? x * cs[i] + y * sn[i] : x * cs[i] - y * sn[i];
+            }
+        }
+        if (query) {
+            q_dst[e] = from_float<T>(x);
+        } else {
+            k_dst[e - H * Dp] = from_float<T>(x);
+            v_dst[e - H * Dp] = from_float<T>(raw);
+        }
+    }
+}
+
+extern "C" int pl_wide_prepare(const float* rows, const float* bias, int stride, int off, int normed, float eps,
+                               const float* q_gain, const float* k_gain, const float* freq, int rot, const int* positions,
+                               const int* seq_of, const int* block_table, int max_blocks, int block_size, int write_kv,
+                               void* q_out, void* k_pool, void* v_pool, int dtype, int n, int H, int G, int D, int Dp,
+                               hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && H > 0 && G > 0 && H % G == 0, "wide_prepare: rows %d, %d query heads over %d key heads", n, H, G);
+    PL_REQUIRE(D > 0 && Dp >= D && Dp <= 1024, "wide_prepare: heads of %d in rows of %d (up to 1024)", D, Dp);
+    PL_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= D && (rot == 0 || freq != nullptr),
+               "wide_prepare: a rotation over %d values of a head of %d", rot, D);
+    PL_REQUIRE(block_size > 0 && max_blocks > 0 && stride >= off + (H + G) * D, "wide_prepare: pages of %d, tables of %d, rows of %d values for %d from %d on",
+               block_size, max_blocks, stride, (H + G) * D, off);
+    const size_t lds = (static_cast<size_t>(H + G) * D + rot) * sizeof(float);
+    PL_REQUIRE(lds <= 64 * 1024, "wide_prepare: %d + %d heads of %d are more than a workgroup's 64 KB hold", H, G, D);
+    if (n == 0) return 0;
+    WidePrepareArgs a{rows, bias, stride, off, normed, eps, q_gain, k_gain, freq, rot, positions, seq_of, block_table,
+                      max_blocks, block_size, write_kv, q_out, k_pool, v_pool, H, G, D, Dp};
+    if (dtype == PL_DTYPE_F32) wide_prepare_kernel<float><<<n, 256, lds, stream>>>(a);
+    else if (dtype == PL_DTYPE_BF16) wide_prepare_kernel<bf16_t><<<n, 256, lds, stream>>>(a);
+    else PL_REQUIRE(false, "wide_prepare: dtype code %d", dtype);
+    PL_CHECK_LAUNCH("wide_prepare");
+    return 0;
+}
+
 struct LatentPrepareArgs {
     const float* rows;        // [n, stride]
     int stride;

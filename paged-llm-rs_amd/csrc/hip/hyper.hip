@@ -236,16 +236,28 @@ struct MoeArgs {
     void* h;               // [n, top, F]
     float* out;            // [n, W]
     int n, W, F, E, top, vocab, act;
+    // Where a router has chosen (null: the table decides and every choice counts 1/top): the expert of pair
+    // (t, c) is choice[t * top + c], -1 for none, E .. E + identity - 1 for an identity expert, whose output is the
+    // row itself; weight[t * top + c] is what the pair counts.
+    const int* choice;
+    const float* weight;
+    int identity;
 };
+
+// The expert of pair (t, c), or -1: the router's choice, or the table's row of the token's id.
+__device__ __forceinline__ int moe_pair_expert(const MoeArgs& a, int t, int c) {
+    if (a.choice != nullptr) return a.choice[static_cast<size_t>(t) * a.top + c];
+    const int id = moe_token(a.ids, a.src, a.fed, t);
+    if (id < 0 || id >= a.vocab) return -1;
+    return a.table[static_cast<size_t>(id) * a.top + c];
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void moe_up_kernel(MoeArgs a) {
     extern __shared__ float moe_x[];
     const int t = blockIdx.x / a.top, c = blockIdx.x % a.top;
     if (a.positions[t] < 0) return;
-    const int id = moe_token(a.ids, a.src, a.fed, t);
-    if (id < 0 || id >= a.vocab) return;
-    const int e = a.table[static_cast<size_t>(id) * a.top + c];
+    const int e = moe_pair_expert(a, t, c);
     if (e < 0 || e >= a.E) return;
     const int W = a.W, F = a.F;
     const T* x = static_cast<const T*>(a.x) + static_cast<size_t>(t) * W;
@@ -269,11 +281,12 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeArgs a) {
     const int W = a.W, F = a.F, top = a.top;
     float* o = a.out + static_cast<size_t>(t) * W;
     const int lane = threadIdx.x % PL_WAVE, wave = threadIdx.x / PL_WAVE, waves = blockDim.x / PL_WAVE;
-    const int id = a.positions[t] < 0 ? -1 : moe_token(a.ids, a.src, a.fed, t);
+    const int id = a.positions[t] < 0 ? -1 : (a.choice != nullptr ? 0 : moe_token(a.ids, a.src, a.fed, t));
     if (id < 0 || id >= a.vocab) {
         for (int w = blockIdx.y * blockDim.x + threadIdx.x; w < W; w += gridDim.y * blockDim.x) o[w] = 0.f;
         return;
     }
+    const T* x = static_cast<const T*>(a.x) + static_cast<size_t>(t) * W;
     const T* h = static_cast<const T*>(a.h) + static_cast<size_t>(t) * top * F;
     for (int k = threadIdx.x; k < top * F; k += blockDim.x) moe_h[k] = to_float(h[k]);
     __syncthreads();
@@ -281,10 +294,12 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeArgs a) {
     for (int w = blockIdx.y * waves + wave; w < W; w += gridDim.y * waves) {
         float sum = 0.f;
         for (int c = 0; c < top; ++c) {
-            const int e = a.table[static_cast<size_t>(id) * top + c];
+            const int e = moe_pair_expert(a, t, c);
+            const float counts = a.weight != nullptr ? a.weight[static_cast<size_t>(t) * top + c] : share;
+            if (e >= a.E && e < a.E + a.identity) sum += to_float(x[w]) * counts;
             if (e < 0 || e >= a.E) continue;
             const T* down = static_cast<const T*>(a.w_down) + (static_cast<size_t>(e) * W + w) * F;
-            sum += moe_dot<T>(down, moe_h + c * F, F, lane) * share;
+            sum += moe_dot<T>(down, moe_h + c * F, F, lane) * counts;
         }
         if (lane == 0) o[w] = sum;
     }
@@ -292,16 +307,20 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeArgs a) {
 
 // out[t] (32-bit) = (1/top) sum over the experts e that table[id of t] names of down_e (act(gate_e x_t) * (up_e x_t)).
 // x [n, W], w_gu [E, 2 F, W], w_down [E, W, F] and the workspace h [n, top, F] in `dtype`; table [vocab, top].
+// With `choice` [n, top] (and `weight` [n, top]) a router has chosen instead of the table: see MoeArgs.
 extern "C" int pl_moe_rows(const void* x, const int* ids, const int* src, const int* fed, const int* positions,
                            const int* table, const void* w_gu, const void* w_down, void* h, float* out, int dtype,
-                           int n, int W, int F, int E, int top, int vocab, int act, hipStream_t stream) {
-    PL_REQUIRE(n >= 0 && W > 0 && F > 0 && E > 0 && top > 0 && top <= E && vocab > 0 && act >= 0 && act <= 2,
+                           int n, int W, int F, int E, int top, int vocab, int act, const int* choice, const float* weight,
+                           int identity, hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && W > 0 && F > 0 && E > 0 && top > 0 && top <= E + identity && identity >= 0 && vocab > 0 && act >= 0 && act <= 2,
                "moe_rows: %d rows of %d, %d experts of %d, %d a row", n, W, E, F, top);
+    PL_REQUIRE((choice != nullptr) != (table != nullptr) && (weight == nullptr || choice != nullptr),
+               "moe_rows: the experts of a row are a table's or a router's");
     PL_REQUIRE((src == nullptr) == (fed == nullptr), "moe_rows: rows fed from the step before need both the rows and the tokens");
     PL_REQUIRE(W <= 16384 && static_cast<long long>(top) * F <= 16384, "moe_rows: rows of %d, %d experts of %d a row", W, top, F);
     PL_REQUIRE(static_cast<long long>(n) * top < (1ll << 31), "moe_rows: %d rows", n);
     if (n == 0) return 0;
-    MoeArgs a{x, ids, src, fed, positions, table, w_gu, w_down, h, out, n, W, F, E, top, vocab, act};
+    MoeArgs a{x, ids, src, fed, positions, table, w_gu, w_down, h, out, n, W, F, E, top, vocab, act, choice, weight, identity};
     // few rows: deal an expert's rows of weights to several workgroups, so that the chip has work
     const int cu = pl_compute_units();
     int up_parts = 1, down_parts = 1;
@@ -329,7 +348,7 @@ extern "C" int pl_moe_rows(const void* x, const int* ids, const int* src, const 
 // tile_group[i] = the expert of tile i (or -1 behind the last).  Which of an expert's pairs gets which of
 // its slots is left to the order in which the threads arrive: nothing computed from a slot depends on it.
 __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* ids, const int* src, const int* fed, const int* positions,
-                                                        const int* table, int n, int top, int E, int vocab, int tile,
+                                                        const int* table, const int* choice, int n, int top, int E, int vocab, int tile,
                                                         int tiles, int* gather, int* slot_of, int* tile_group) {
     extern __shared__ int moe_counts[];               // count [E], base [E], cursor [E]
     int* count = moe_counts;
@@ -342,9 +361,14 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* ids, const in
     auto expert_of = [&](int p) -> int {
         const int t = p / top;
         if (positions[t] < 0) return -1;
-        const int id = moe_token(ids, src, fed, t);
-        if (id < 0 || id >= vocab) return -1;
-        const int e = table[static_cast<size_t>(id) * top + (p - t * top)];
+        int e;
+        if (choice != nullptr) {
+            e = choice[p];                            // (an identity expert, E or beyond, takes no slot)
+        } else {
+            const int id = moe_token(ids, src, fed, t);
+            if (id < 0 || id >= vocab) return -1;
+            e = table[static_cast<size_t>(id) * top + (p - t * top)];
+        }
         return (e >= 0 && e < E) ? e : -1;
     };
     for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
@@ -376,14 +400,15 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* ids, const in
 }
 
 // tiles: what the caller has room for, at least ceil(n * top / tile) + min(E, n * top).
-extern "C" int pl_moe_sort(const int* ids, const int* src, const int* fed, const int* positions, const int* table, int n,
-                           int top, int E, int vocab, int tile, int tiles, int* gather, int* slot_of, int* tile_group,
-                           hipStream_t stream) {
-    PL_REQUIRE(n > 0 && top > 0 && E > 0 && E <= 4096 && top <= E && vocab > 0 && tile > 0, "moe_sort: %d rows, %d of %d experts", n, top, E);
+extern "C" int pl_moe_sort(const int* ids, const int* src, const int* fed, const int* positions, const int* table,
+                           const int* choice, int n, int top, int E, int vocab, int tile, int tiles, int* gather, int* slot_of,
+                           int* tile_group, hipStream_t stream) {
+    PL_REQUIRE(n > 0 && top > 0 && E > 0 && E <= 4096 && vocab > 0 && tile > 0, "moe_sort: %d rows, %d of %d experts", n, top, E);
+    PL_REQUIRE((choice != nullptr) != (table != nullptr), "moe_sort: the experts of a row are a table's or a router's");
     PL_REQUIRE(static_cast<long long>(n) * top < (1ll << 30) && tiles >= (n * top + tile - 1) / tile + (E < n * top ? E : n * top),
                "moe_sort: %d tiles of %d for %d rows with %d of %d experts", tiles, tile, n, top, E);
     PL_REQUIRE((src == nullptr) == (fed == nullptr), "moe_sort: rows fed from the step before need both the rows and the tokens");
-    moe_sort_kernel<<<1, 1024, 3 * E * sizeof(int), stream>>>(ids, src, fed, positions, table, n, top, E, vocab, tile, tiles,
+    moe_sort_kernel<<<1, 1024, 3 * E * sizeof(int), stream>>>(ids, src, fed, positions, table, choice, n, top, E, vocab, tile, tiles,
                                                                gather, slot_of, tile_group);
     PL_CHECK_LAUNCH("moe_sort");
     return 0;
@@ -392,15 +417,29 @@ extern "C" int pl_moe_sort(const int* ids, const int* src, const int* fed, const
 // out[t, :] = (1/top) sum over c of y[slot_of[t * top + c], :], the choices in their order; a pair without a slot adds nothing.
 // y may come in `splits` copies, `split_stride` floats apart, each a stretch of the product's inner width: a pair's
 // copies are added in their order.
+// With `weight` a pair counts weight[t * top + c] instead of 1/top, and a pair whose `choice` is E or beyond (an
+// identity expert) adds the row of x itself (of type `x_dtype`) with its weight.
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ slot_of,
-                                                          float* __restrict__ out, int top, int W, int splits, size_t split_stride) {
+                                                          float* __restrict__ out, int top, int W, int splits, size_t split_stride,
+                                                          const float* __restrict__ weight, const int* __restrict__ choice,
+                                                          const void* __restrict__ x, int x_dtype, int E) {
     const int t = blockIdx.x;
-    const float share = 1.f / static_cast<float>(top);
+    const float even = 1.f / static_cast<float>(top);
     for (int w = threadIdx.x * 4; w < W; w += blockDim.x * 4) {
         float4 sum = {0.f, 0.f, 0.f, 0.f};
         for (int c = 0; c < top; ++c) {
             const int slot = slot_of[t * top + c];
-            if (slot < 0) continue;
+            const float share = weight != nullptr ? weight[t * top + c] : even;
+            if (slot < 0) {
+                if (choice != nullptr && choice[t * top + c] >= E) {
+                    const size_t at = static_cast<size_t>(t) * W + w;
+                    sum.x += load_as_float(x, x_dtype, at) * share;
+                    sum.y += load_as_float(x, x_dtype, at + 1) * share;
+                    sum.z += load_as_float(x, x_dtype, at + 2) * share;
+                    sum.w += load_as_float(x, x_dtype, at + 3) * share;
+                }
+                continue;
+            }
             float4 v = *reinterpret_cast<const float4*>(y + static_cast<size_t>(slot) * W + w);
             for (int s = 1; s < splits; ++s) {
                 const float4 more = *reinterpret_cast<const float4*>(y + s * split_stride + static_cast<size_t>(slot) * W + w);
@@ -419,10 +458,142 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 }
 
 extern "C" int pl_moe_combine(const float* y, const int* slot_of, float* out, int n, int top, int W, int splits,
-                              long long split_stride, hipStream_t stream) {
+                              long long split_stride, const float* weight, const int* choice, const void* x, int x_dtype,
+                              int E, hipStream_t stream) {
     PL_REQUIRE(n >= 0 && top > 0 && W > 0 && W % 4 == 0 && splits >= 1, "moe_combine: %d rows of %d, %d a row, %d copies", n, W, top, splits);
+    PL_REQUIRE(choice == nullptr || (x != nullptr && (x_dtype == PL_DTYPE_F32 || x_dtype == PL_DTYPE_BF16)),
+               "moe_combine: identity experts need the rows they hand through");
     if (n == 0) return 0;
-    moe_combine_kernel<<<n, 256, 0, stream>>>(y, slot_of, out, top, W, splits, static_cast<size_t>(split_stride));
+    moe_combine_kernel<<<n, 256, 0, stream>>>(y, slot_of, out, top, W, splits, static_cast<size_t>(split_stride), weight, choice,
+                                              x, x_dtype, E);
     PL_CHECK_LAUNCH("moe_combine");
+    return 0;
+}
+
+// ---- a router's choice ------------------------------------------------------------------------------------
+
+// The lane that holds the largest value (the lowest index among equals) learns nothing special: every lane gets
+// (value, index) of the winner.
+__device__ __forceinline__ void wave_best(float& v, int& i) {
+#pragma unroll
+    for (int off = PL_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(v, off, PL_WAVE);
+        const int oi = __shfl_xor(i, off, PL_WAVE);
+        if (ov > v || (ov == v && oi < i)) {
+            v = ov;
+            i = oi;
+        }
+    }
+}
+
+// A wave a row.  z [n, stride] are the router's 32-bit logits over `total` outputs.  s = softmax(z); the choice goes
+// by s + correction; outputs form `groups` equal groups of neighbours, a group counts by its largest choice score and
+// only members of the `kept` best groups can be chosen (the others count as minus infinity); the `top` largest are
+// chosen (the lower index among equals), in that order; a chosen output weighs s, divided, with `normalised`, by the
+// chosen ones' sum plus weight_eps.  Rows at position -1 choose nothing (-1, weight 0).
+__global__ __launch_bounds__(64) void router_select_kernel(const float* __restrict__ z, int stride, const float* __restrict__ correction,
+                                                           const int* __restrict__ positions, int total, int top, int groups,
+                                                           int kept, int normalised, float weight_eps, int* __restrict__ choice,
+                                                           float* __restrict__ weight) {
+    extern __shared__ float router_lds[];             // score [total], choice score [total], group score [groups], kept or not [groups]
+    float* score = router_lds;
+    float* pick = router_lds + total;
+    float* group = pick + total;
+    float* stays = group + groups;
+    const int t = blockIdx.x, lane = threadIdx.x;
+    int* chosen = choice + static_cast<size_t>(t) * top;
+    float* counts = weight + static_cast<size_t>(t) * top;
+    if (positions != nullptr && positions[t] < 0) {
+        for (int c = lane; c < top; c += PL_WAVE) {
+            chosen[c] = -1;
+            counts[c] = 0.f;
+        }
+        return;
+    }
+    const float* row = z + static_cast<size_t>(t) * stride;
+    float largest = -INFINITY;
+    for (int e = lane; e < total; e += PL_WAVE) largest = fmaxf(largest, row[e]);
+    largest = wave_max(largest);
+    float sum = 0.f;
+    for (int e = lane; e < total; e += PL_WAVE) {
+        const float x = expf(row[e] - largest);
+        score[e] = x;
+        sum += x;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < total; e += PL_WAVE) {
+        const float s = score[e] / sum;
+        score[e] = s;
+        pick[e] = correction != nullptr ? s + correction[e] : s;
+    }
+    __syncthreads();
+    if (groups > 1) {
+        const int size = total / groups;
+        for (int g = lane; g < groups; g += PL_WAVE) {
+            float best = -INFINITY;
+            for (int e = g * size; e < (g + 1) * size; ++e) best = fmaxf(best, pick[e]);
+            group[g] = best;
+        }
+        __syncthreads();
+        // the best `kept` groups keep their members, the others' members leave
+        for (int g = lane; g < groups; g += PL_WAVE) stays[g] = 0.f;
+        __syncthreads();
+        for (int k = 0; k < kept; ++k) {
+            float v = -INFINITY;
+            int at = 0x7fffffff;
+            for (int g = lane; g < groups; g += PL_WAVE) {
+                const float x = group[g];
+                if (stays[g] == 0.f && (at == 0x7fffffff || x > v)) {
+                    v = x;
+                    at = g;
+                }
+            }
+            wave_best(v, at);
+            if (lane == 0 && at != 0x7fffffff) stays[at] = 1.f;
+            __syncthreads();
+        }
+        for (int e = lane; e < total; e += PL_WAVE)
+            if (stays[e / size] == 0.f) pick[e] = -INFINITY;
+        __syncthreads();
+    }
+    float chosen_sum = 0.f;
+    for (int c = 0; c < top; ++c) {
+        float v = -INFINITY;
+        int at = 0x7fffffff;
+        for (int e = lane; e < total; e += PL_WAVE) {
+            const float x = pick[e];
+            if (!isnan(x) && (x > v || (x == v && e < at))) {
+                v = x;
+                at = e;
+            }
+        }
+        wave_best(v, at);
+        if (at == 0x7fffffff) at = -1;               // (nothing left to choose from)
+        const float s = at >= 0 ? score[at] : 0.f;
+        chosen_sum += s;
+        if (lane == 0) {
+            chosen[c] = at;
+            counts[c] = s;
+            if (at >= 0) pick[at] = NAN;             // (taken: below every other value, minus infinity included)
+        }
+        __syncthreads();
+    }
+    if (normalised) {
+        for (int c = lane; c < top; c += PL_WAVE) counts[c] = counts[c] / (chosen_sum + weight_eps);
+    }
+}
+
+extern "C" int pl_router_select(const float* z, int stride, const float* correction, const int* positions, int n, int total,
+                                int top, int groups, int kept, int normalised, float weight_eps, int* choice, float* weight,
+                                hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && total > 0 && total <= 8192 && stride >= total && top > 0 && top <= total,
+               "router_select: %d rows, %d of %d outputs in rows of %d", n, top, total, stride);
+    PL_REQUIRE(groups >= 1 && total % groups == 0 && kept >= 1 && kept <= groups && top <= kept * (total / groups),
+               "router_select: %d outputs in %d groups of which %d are kept, %d chosen", total, groups, kept, top);
+    if (n == 0) return 0;
+    const size_t lds = 2 * (static_cast<size_t>(total) + groups) * sizeof(float);
+    router_select_kernel<<<n, 64, lds, stream>>>(z, stride, correction, positions, total, top, groups, kept, normalised, weight_eps,
+                                                 choice, weight);
+    PL_CHECK_LAUNCH("router_select");
     return 0;
 }

@@ -78,9 +78,12 @@ def _signatures(lib) -> None:
         "pl_hc_step": [p, p, p, p, p, p, f, p, i, p, i, i, i, p],
         "pl_stream_copies": [p, p, i, i, i, p],
         "pl_softcap": [p, f, ctypes.c_long, p],
-        "pl_moe_rows": [p, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, p],
-        "pl_moe_sort": [p, p, p, p, p, i, i, i, i, i, i, p, p, p, p],
-        "pl_moe_combine": [p, p, p, i, i, i, i, ctypes.c_longlong, p],
+        "pl_moe_rows": [p, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, p, p, i, p],
+        "pl_moe_sort": [p, p, p, p, p, p, i, i, i, i, i, i, p, p, p, p],
+        "pl_moe_combine": [p, p, p, i, i, i, i, ctypes.c_longlong, p, p, p, i, i, p],
+        "pl_router_select": [p, i, p, p, i, i, i, i, i, i, f, p, p, p],
+        "pl_wide_prepare": [p, p, i, i, i, f, p, p, p, i, p, p, p, i, i, i, p, p, p, i, i, i, i, i, i, p],
+        "pl_parallel_step": [p, p, p, p, p, p, p, p, f, p, p, i, p, i, i, p],
         "pl_gemm_tiled_grouped": [p, p, p, p, p, ctypes.c_longlong, i, i, i, i, i, i, i, p],
     }
     for name, argtypes in table.items():
@@ -1534,28 +1537,43 @@ def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
     return x
 
 
-def moe_rows(x: torch.Tensor, batch, table: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
-             activation: str = "silu") -> torch.Tensor:
+def _routed(n: int, E: int, choice, weight, identity: int) -> int:
+    """Checks a router's choice for ``n`` rows ([n, top] int32, with weights [n, top] 32-bit) and gives ``top``."""
+    _need(choice, "chosen experts", None, torch.int32)
+    if choice.dim() != 2 or choice.shape[0] != n or not 1 <= choice.shape[1] <= E + identity or identity < 0:
+        raise TensorError(f"chosen experts of shape {tuple(choice.shape)} for {n} rows and {E} + {identity} experts")
+    _need(weight, "weights of the chosen experts", tuple(choice.shape), torch.float32)
+    return choice.shape[1]
+
+
+def moe_rows(x: torch.Tensor, batch, table, w_gate_up: torch.Tensor, w_down: torch.Tensor,
+             activation: str = "silu", choice=None, weight=None, identity: int = 0) -> torch.Tensor:
     """Experts chosen by a table over token ids, a row at a time: 32-bit [n, W], row t the mean over the experts e
     that ``table[id of t]`` names of down_e (act(gate_e x_t) * (up_e x_t)).  ``w_gate_up`` [E, 2 F, W] (an expert's
     gate rows, then its up rows), ``w_down`` [E, W, F], of ``x``'s type; ``table`` [vocabulary, top] int32.  A row's
-    id is the batch's, or the one an earlier step left on the device; padding rows give zeros."""
+    id is the batch's, or the one an earlier step left on the device; padding rows give zeros.
+    With ``choice`` and ``weight`` ([n, top]; no table) a router has chosen: pair (t, c) runs expert choice[t, c] and
+    counts weight[t, c]; a choice of E .. E + ``identity`` - 1 is an identity expert, whose output is the row itself;
+    -1 is none."""
     n, W = x.shape
     _need(x, "rows")
     E, F2, _ = w_gate_up.shape
     F = F2 // 2
     _need(w_gate_up, "gate and up weights of the experts", (E, 2 * F, W), x.dtype)
     _need(w_down, "down weights of the experts", (E, W, F), x.dtype)
-    _need(table, "table of experts", None, torch.int32)
-    vocab, top = table.shape
+    if choice is not None:
+        vocab, top = 1, _routed(n, E, choice, weight, identity)
+    else:
+        _need(table, "table of experts", None, torch.int32)
+        vocab, top = table.shape
     fed = getattr(batch, "fed_tokens", None)
     src = batch.token_src if fed is not None else None
     h = torch.empty((n, top, F), dtype=x.dtype, device=x.device)
     out = torch.empty((n, W), dtype=torch.float32, device=x.device)
     _check(library().pl_moe_rows(x.data_ptr(), batch.token_ids.data_ptr(), _ptr(src), _ptr(fed),
-                                 batch.positions.data_ptr(), table.data_ptr(), w_gate_up.data_ptr(), w_down.data_ptr(),
+                                 batch.positions.data_ptr(), _ptr(table), w_gate_up.data_ptr(), w_down.data_ptr(),
                                  h.data_ptr(), out.data_ptr(), _code(x, "rows"), n, W, F, E, top, vocab,
-                                 activation_code(activation), _stream()))
+                                 activation_code(activation), _ptr(choice), _ptr(weight), int(identity), _stream()))
     return out
 
 
@@ -1578,8 +1596,8 @@ def moe_down_splits(tiles: int, width: int, ff: int) -> int:
     return splits
 
 
-def moe_grouped(x: torch.Tensor, batch, table: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
-                activation: str = "silu") -> torch.Tensor:
+def moe_grouped(x: torch.Tensor, batch, table, w_gate_up: torch.Tensor, w_down: torch.Tensor,
+                activation: str = "silu", choice=None, weight=None, identity: int = 0) -> torch.Tensor:
     """What ``moe_rows`` computes, with the step's (row, choice) pairs dealt to their experts first: an expert's
     pairs fill tiles of 128 rows, and two grouped products on the matrix cores (gate and up with the activation
     behind them; down with 32-bit sums out) read an expert's weights once a tile.  A last pass adds a row's
@@ -1591,8 +1609,11 @@ def moe_grouped(x: torch.Tensor, batch, table: torch.Tensor, w_gate_up: torch.Te
     F = F2 // 2
     _need(w_gate_up, "gate and up weights of the experts", (E, 2 * F, W), x.dtype)
     _need(w_down, "down weights of the experts", (E, W, F), x.dtype)
-    _need(table, "table of experts", None, torch.int32)
-    vocab, top = table.shape
+    if choice is not None:
+        vocab, top = 1, _routed(n, E, choice, weight, identity)
+    else:
+        _need(table, "table of experts", None, torch.int32)
+        vocab, top = table.shape
     out = torch.empty((n, W), dtype=torch.float32, device=x.device)
     if n == 0:
         return out
@@ -1605,8 +1626,9 @@ def moe_grouped(x: torch.Tensor, batch, table: torch.Tensor, w_gate_up: torch.Te
     lib, stream = library(), _stream()
     ints = torch.empty((slots + pairs + tiles,), dtype=torch.int32, device=x.device)
     gather, slot_of, tile_group = ints[:slots], ints[slots:slots + pairs], ints[slots + pairs:]
-    _check(lib.pl_moe_sort(batch.token_ids.data_ptr(), _ptr(src), _ptr(fed), batch.positions.data_ptr(), table.data_ptr(),
-                           n, top, E, vocab, MOE_TILE, tiles, gather.data_ptr(), slot_of.data_ptr(), tile_group.data_ptr(), stream))
+    _check(lib.pl_moe_sort(batch.token_ids.data_ptr(), _ptr(src), _ptr(fed), batch.positions.data_ptr(), _ptr(table),
+                           _ptr(choice), n, top, E, vocab, MOE_TILE, tiles, gather.data_ptr(), slot_of.data_ptr(),
+                           tile_group.data_ptr(), stream))
     hidden = torch.empty((slots, F), dtype=torch.bfloat16, device=x.device)
     _check(lib.pl_gemm_tiled_grouped(x.data_ptr(), w_gate_up.data_ptr(), hidden.data_ptr(), tile_group.data_ptr(),
                                      gather.data_ptr(), 2 * F * W, tiles, n, F, W, 1, activation_code(activation), 1, stream))
@@ -1614,5 +1636,98 @@ def moe_grouped(x: torch.Tensor, batch, table: torch.Tensor, w_gate_up: torch.Te
     y = torch.empty((splits, slots, W), dtype=torch.float32, device=x.device)
     _check(lib.pl_gemm_tiled_grouped(hidden.data_ptr(), w_down.data_ptr(), y.data_ptr(), tile_group.data_ptr(), 0,
                                      W * F, tiles, slots, W, F, 3, 0, splits, stream))
-    _check(lib.pl_moe_combine(y.data_ptr(), slot_of.data_ptr(), out.data_ptr(), n, top, W, splits, slots * W, stream))
+    _check(lib.pl_moe_combine(y.data_ptr(), slot_of.data_ptr(), out.data_ptr(), n, top, W, splits, slots * W,
+                              _ptr(weight), _ptr(choice), x.data_ptr(), _code(x, "rows"), E, stream))
     return out
+
+
+def router_select(logits: torch.Tensor, correction, positions, top: int, groups: int = 1, kept: int = 1,
+                  normalised: bool = True, weight_eps: float = 1e-20):
+    """A router's choice for every row of its 32-bit ``logits`` [n, outputs]: (chosen [n, top] int32, weights [n, top]
+    32-bit).  Scores are the softmax over all outputs; the choice goes by score plus ``correction`` ([outputs] 32-bit, or
+    None); outputs form ``groups`` equal groups of neighbours, a group counts by its best choice score, and only members
+    of the best ``kept`` groups can be chosen; the ``top`` largest are chosen, the lower index among equals; a chosen
+    output weighs its score, divided (``normalised``) by the chosen scores' sum plus ``weight_eps``.  Rows at
+    position -1 choose nothing (-1)."""
+    _need(logits, "router logits", None, torch.float32)
+    if logits.dim() != 2:
+        raise TensorError(f"router logits of shape {tuple(logits.shape)}")
+    n, total = logits.shape
+    if correction is not None:
+        _need(correction, "correction of the choice", (total,), torch.float32)
+    if positions is not None:
+        _need(positions, "positions", (n,), torch.int32)
+    choice = torch.empty((n, top), dtype=torch.int32, device=logits.device)
+    weight = torch.empty((n, top), dtype=torch.float32, device=logits.device)
+    _check(library().pl_router_select(logits.data_ptr(), total, _ptr(correction), _ptr(positions), n, total, int(top),
+                                      int(groups), int(kept), 1 if normalised else 0, float(weight_eps),
+                                      choice.data_ptr(), weight.data_ptr(), _stream()))
+    return choice, weight
+
+
+# ---- values that are the keys, q and k normed over all their heads; sublayers side by side ----------------------
+
+def wide_prepare(rows: torch.Tensor, off: int, batch, kv, q_out: torch.Tensor, H: int, G: int, D: int, padded: int,
+                 norm_eps: float | None = None, q_gain=None, k_gain=None, freq=None, rot: int = 0,
+                 write_kv: bool = True, bias: torch.Tensor | None = None) -> None:
+    """Between an attention layer's projections and the attention kernels, for a layer without a value projection:
+    ``rows`` [n, >= off + H D + G D] (32-bit) holds q | k from column ``off``; ``bias`` ([H D + G D] 32-bit) is added
+    first.  The values are the keys as they stand then.  q is divided by its root mean square over ALL its H D
+    values and k over all its G D (``norm_eps``; times a gain a column, [H D] and [G D]); the first ``rot`` values of every
+    head turn in pairs (2i, 2i + 1) by position * ``freq``[i] (32-bit).  q goes to ``q_out`` [n, H * padded], the keys and
+    the values into the pages, every head in ``padded`` values with zeros behind its own."""
+    n = rows.shape[0]
+    _need(rows, "projected rows", None, torch.float32)
+    if rows.dim() != 2:
+        raise TensorError(f"projected rows of shape {tuple(rows.shape)}")
+    _need(q_out, "query buffer", (n, H * padded))
+    for pool, what in ((kv.k_pool, "key pool"), (kv.v_pool, "value pool")):
+        _need(pool, what, None, q_out.dtype)
+        if pool.dim() != 2 or pool.shape[1] != G * padded or pool.shape[0] % kv.block_size:
+            raise TensorError(f"{what} has shape {tuple(pool.shape)}, expected [pages*{kv.block_size}, {G * padded}]")
+    if q_gain is not None:
+        _need(q_gain, "query gain", (H * D,), torch.float32)
+    if k_gain is not None:
+        _need(k_gain, "key gain", (G * D,), torch.float32)
+    if rot:
+        _need(freq, "rotation frequencies", (rot // 2,), torch.float32)
+    if bias is not None:
+        _need(bias, "biases of q and k", (H * D + G * D,), torch.float32)
+    _check(library().pl_wide_prepare(
+        rows.data_ptr(), _ptr(bias), rows.shape[1], int(off), 1 if norm_eps is not None else 0, float(norm_eps or 0.0),
+        _ptr(q_gain), _ptr(k_gain), _ptr(freq) if rot else 0, int(rot), batch.positions.data_ptr(), batch.seq_of.data_ptr(),
+        kv.block_table.data_ptr(), kv.block_table.shape[1], kv.block_size, 1 if write_kv else 0, q_out.data_ptr(),
+        kv.k_pool.data_ptr(), kv.v_pool.data_ptr(), _code(q_out, "query buffer"), n, H, G, D, padded, _stream()))
+
+
+def parallel_step(resid: torch.Tensor, a=None, ls1=None, b=None, ls2=None, more=None, gain1=None, gain2=None,
+                  eps: float = 0.0, out_dtype: torch.dtype = torch.float32, rows=None):
+    """One pass over the rows of the 32-bit stream for a layer whose sublayers stand side by side, either half
+    optional.  Sums: resid += ls1 * a + ls2 * b + more (``a``, ``b``, ``more`` [n, W] 32-bit; ``ls1``, ``ls2`` [W] 32-bit
+    or None for ones), in place.  Norms of the updated rows: rms-normed rows times ``gain1`` and, where given, times
+    ``gain2`` (both [W] 32-bit), in ``out_dtype``; (rows1, rows2), each None where its gain is.  ``rows``: the rows to
+    norm (then nothing is summed)."""
+    _need(resid, "residual stream", None, torch.float32)
+    if resid.dim() != 2:
+        raise TensorError(f"a stream of shape {tuple(resid.shape)}")
+    n, W = resid.shape
+    for t, what in ((a, "first sublayer's output"), (b, "second sublayer's output"), (more, "rows to add")):
+        if t is not None:
+            _need(t, what, (n, W), torch.float32)
+    for t, what in ((ls1, "first layer scale"), (ls2, "second layer scale"), (gain1, "first norm gain"), (gain2, "second norm gain")):
+        if t is not None:
+            _need(t, what, (W,), torch.float32)
+    if (ls1 is not None and a is None) or (ls2 is not None and b is None) or (gain2 is not None and gain1 is None):
+        raise TensorError("a layer scale without its sublayer's output, or a second norm without a first")
+    count = n
+    if rows is not None:
+        _need(rows, "rows to norm", None, torch.int32)
+        count = rows.numel()
+    out1 = torch.empty((count, W), dtype=out_dtype, device=resid.device) if gain1 is not None else None
+    out2 = torch.empty((count, W), dtype=out_dtype, device=resid.device) if gain2 is not None else None
+    if a is None and b is None and more is None and gain1 is None:
+        return None, None
+    _check(library().pl_parallel_step(resid.data_ptr(), _ptr(a), _ptr(ls1), _ptr(b), _ptr(ls2), _ptr(more), _ptr(gain1),
+                                      _ptr(gain2), float(eps), _ptr(out1), _ptr(out2), _CODES[out_dtype], _ptr(rows),
+                                      count, W, _stream()))
+    return out1, out2

@@ -431,3 +431,114 @@ class HyperConnectionBlock:
 
 
 register_block("hyper_connections", HyperConnectionBlock)
+
+
+class PendingSums:
+    """What a layer whose sublayers stand side by side has not added to the stream yet: its sublayers' 32-bit outputs
+    and their gains a column.  The layer behind adds them in the pass that norms its own rows."""
+
+    __slots__ = ("a", "ls1", "b", "ls2")
+    filled = True            # (what a layer hands to the next is looked at only when it says it holds something)
+
+    def __init__(self, a, ls1, b, ls2):
+        self.a, self.ls1, self.b, self.ls2 = a, ls1, b, ls2
+
+
+class ParallelBlock:
+    """The arrangement whose sublayers read the same stream through a norm each: with a = norm1(x) and b = norm2(x),
+    x <- x + ls1 * mixer(a) + ls2 * feed_forward(b).  ``LayerSpec.layer_scale`` says whether the gains a column ls1 and
+    ls2 exist (tensors ``ls1``, ``ls2``); without it the outputs are added as they are.  A layer whose spec has no
+    feed-forward adds the mixer's output only (``norm2`` and ``ls2``, if a checkpoint carries them, are not used).
+
+    The stream and every sum into it are 32-bit; sublayers hand back 32-bit rows.  One kernel adds a layer's two outputs
+    into the stream and norms the next layer's two rows in the same pass (``kernels.parallel_step``): a layer that is
+    followed by another of this arrangement leaves its sums to that layer's pass (``PendingSums``), so a layer is one
+    pass over the stream.  ``ctx.stream_addend`` (rows the decoder wants added to the stream before this run) joins
+    that pass too.  Tensor names: the norms' gains under the norms' own names."""
+
+    NAMES = {"norm1": "norm1", "mixer": "mix", "norm2": "norm2", "feed_forward": "mlp", "scale1": "ls1", "scale2": "ls2"}
+    # the decoder may hand this block rows to add to the stream before it runs (``LayerContext.stream_addend``)
+    takes_stream_addend = True
+
+    @classmethod
+    def names_of(cls, layer) -> dict:
+        given = getattr(layer, "names", None) or {}
+        unknown = sorted(set(given) - set(cls.NAMES))
+        if unknown:
+            raise ConfigError(f"a layer names members that this arrangement does not have: {unknown}")
+        return {**cls.NAMES, **given}
+
+    @classmethod
+    def declare(cls, layer, hidden: int) -> list:
+        from ..weights.loader import ParamDecl
+
+        n = cls.names_of(layer)
+        mixer = lookup(MIXERS, layer.mixer.kind, "mixer")
+        gain = lookup(NORMS, layer.norm.kind, "norm").declare(layer.norm, hidden)[0].role
+        scaled = bool(getattr(layer, "layer_scale", False))
+        has_ffn = layer.feed_forward is not None
+        decls = [ParamDecl(n["norm1"], (hidden,), gain), ParamDecl(n["norm2"], (hidden,), gain, optional=not has_ffn)]
+        decls += prefixed(mixer.declare(layer.mixer, hidden), n["mixer"])
+        if has_ffn:
+            ffn = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")
+            decls += prefixed(ffn.declare(layer.feed_forward, hidden), n["feed_forward"])
+        if scaled:
+            decls += [ParamDecl(n["scale1"], (hidden,), "gain"), ParamDecl(n["scale2"], (hidden,), "gain", optional=not has_ffn)]
+        return decls
+
+    def __init__(self, layer, hidden: int, params: dict, dtype, device, shared: dict):
+        n = self.names = self.names_of(layer)
+        norm = lookup(NORMS, layer.norm.kind, "norm")
+        if not getattr(norm, "fuses_into_product", False):
+            raise ConfigError(f"norm {layer.norm.kind!r} cannot run inside the pass over the stream of a layer whose "
+                              "sublayers stand side by side (it needs a 32-bit gain and an eps, nothing else)")
+        self.dtype, self.hidden = dtype, hidden
+        self.norm1 = norm(layer.norm, hidden, {"weight": params[n["norm1"]]}, dtype, device)
+        self.norm1.takes_pending_sums = True       # (how the layer before learns that its sums can wait)
+        self.mixer = lookup(MIXERS, layer.mixer.kind, "mixer")(
+            layer.mixer, hidden, scoped(params, n["mixer"]), dtype, device, shared)
+        scaled = bool(getattr(layer, "layer_scale", False))
+        self.ls1 = params[n["scale1"]].to(torch.float32).contiguous() if scaled else None
+        self.norm2 = self.feed_forward = self.ls2 = None
+        if layer.feed_forward is not None:
+            self.norm2 = norm(layer.norm, hidden, {"weight": params[n["norm2"]]}, dtype, device)
+            self.feed_forward = lookup(FEED_FORWARDS, layer.feed_forward.kind, "feed-forward")(
+                layer.feed_forward, hidden, scoped(params, n["feed_forward"]), dtype, device, shared)
+            self.ls2 = params[n["scale2"]].to(torch.float32).contiguous() if scaled else None
+
+    @property
+    def graph_safe(self) -> bool:
+        return getattr(self.mixer, "graph_safe", True) and getattr(self.feed_forward, "graph_safe", True)
+
+    @property
+    def first_norm(self):
+        return self.norm1
+
+    def forward(self, resid, delta, ctx):
+        if delta is not None:
+            kernels.residual_add(resid, delta)
+        before = getattr(ctx, "handed", None)
+        if not isinstance(before, PendingSums):
+            before = PendingSums(None, None, None, None)
+        eps = self.norm1.eps
+        rows1, rows2 = kernels.parallel_step(
+            resid, a=before.a, ls1=before.ls1, b=before.b, ls2=before.ls2, more=getattr(ctx, "stream_addend", None),
+            gain1=self.norm1.gain32, gain2=self.norm2.gain32 if self.norm2 is not None else None, eps=eps,
+            out_dtype=self.dtype)
+        ctx.stream_addend = None
+        mixed = self.mixer.forward(rows1, ctx)
+        out = None
+        if self.feed_forward is not None:
+            ffn = self.feed_forward
+            out = ffn.forward(rows2, batch=ctx.batch) if getattr(ffn, "takes_batch", False) else ffn.forward(rows2)
+            if out.dtype != torch.float32:
+                out = out.float()
+        after = getattr(ctx, "norm_after", None)
+        if ctx.trace is None and after is not None and getattr(after, "takes_pending_sums", False):
+            ctx.handed_out = PendingSums(mixed, self.ls1, out, self.ls2)
+        else:
+            kernels.parallel_step(resid, a=mixed, ls1=self.ls1, b=out, ls2=self.ls2)
+        return None
+
+
+register_block("parallel", ParallelBlock)

@@ -27,7 +27,7 @@ from ..errors import UnsupportedError
 from ..weights.loader import ParamDecl
 from .linear import Linear
 from .registry import register_mixer
-from .rotary import rotary_tables
+from .rotary import rotary_frequencies, rotary_tables
 from .sink_attention import head_sinks
 
 
@@ -86,13 +86,13 @@ class LatentAttention:
         # frequencies alone (rounded from 64-bit), and the kernel multiplies by the position in 32-bit
         self.cos = self.sin = None
         if spec.rotary_turned and spec.max_positions:
+            if getattr(spec, "rotary_scaling", None) is not None:
+                raise UnsupportedError("rescaled rotation frequencies with tables of angles (max_positions = 0 works the angles out)")
             rotary = rotary_tables(PositionSpec("rotary_neighbours", spec.rotary_turned, float(spec.rotary_base),
                                                 int(spec.max_positions)), device, shared)
             self.cos, self.sin = rotary.cos, rotary.sin
         elif spec.rotary_turned:
-            turned = spec.rotary_turned
-            self.cos = torch.tensor([float(spec.rotary_base) ** (-2.0 * i / turned) for i in range(turned // 2)],
-                                    dtype=torch.float64).to(torch.float32).to(device)
+            self.cos = rotary_frequencies(spec.rotary_turned, spec.rotary_base, getattr(spec, "rotary_scaling", None), device)
         self.o_proj = Linear(params["o"])
 
     def cache_spec(self):

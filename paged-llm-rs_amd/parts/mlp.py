@@ -144,3 +144,62 @@ class TableExperts:
 
 
 register_feed_forward("table_experts", TableExperts)
+
+
+class RoutedExperts:
+    """Small gated feed-forwards behind a router, with identity experts behind the real ones: a token's output is the
+    sum over its chosen e of weight_e * expert_e(x), where an identity expert's output is x itself.  The router's
+    logits are one product with 32-bit sums out; scores, the correction for the choice, the groups, the choice and
+    the weights are one kernel in 32-bit (``kernels.router_select``); the chosen pairs then run as the experts by table
+    do: dealt to their experts and multiplied as grouped products on the matrix cores, or a pair at a time.  Nothing
+    depends on the other rows of the step.  The result comes back in 32-bit.
+    Tensors: ``e<i>.gate``, ``e<i>.up`` [ff, width], ``e<i>.down`` [width, ff]; ``router`` [experts + identity, width];
+    ``correction`` [experts + identity]."""
+
+    # forward needs the step (padding rows choose nothing)
+    takes_batch = True
+    graph_safe = True
+
+    @staticmethod
+    def declare(spec, hidden: int) -> list:
+        decls = []
+        for e in range(spec.experts):
+            decls += [ParamDecl(f"e{e}.gate", (spec.intermediate_size, hidden)),
+                      ParamDecl(f"e{e}.up", (spec.intermediate_size, hidden)),
+                      ParamDecl(f"e{e}.down", (hidden, spec.intermediate_size))]
+        total = spec.experts + spec.identity
+        decls.append(ParamDecl("router", (total, hidden), "router"))
+        if spec.corrected:
+            decls.append(ParamDecl("correction", (total,), "bias"))
+        return decls
+
+    def __init__(self, spec, hidden: int, params: dict, dtype, device, shared: dict):
+        if spec.activation not in kernels.ACTIVATIONS:
+            raise UnsupportedError(f"activation {spec.activation!r}, the kernels know {', '.join(sorted(kernels.ACTIVATIONS))}")
+        if spec.score != "softmax":
+            raise UnsupportedError(f"router scores of kind {spec.score!r} (softmax)")
+        E, total = spec.experts, spec.experts + spec.identity
+        if E < 1 or spec.identity < 0 or not 1 <= spec.top <= total:
+            raise UnsupportedError(f"{spec.top} of {E} + {spec.identity} experts a token")
+        if spec.groups < 1 or total % spec.groups or not 1 <= spec.groups_kept <= spec.groups \
+                or spec.top > spec.groups_kept * (total // spec.groups):
+            raise UnsupportedError(f"{total} router outputs in {spec.groups} groups of which {spec.groups_kept} are kept, "
+                                   f"{spec.top} chosen")
+        self.spec, self.activation = spec, spec.activation
+        # [E, 2 F, W]: an expert's gate rows, then its up rows; [E, W, F]
+        self.w_gate_up = torch.stack([torch.cat([params[f"e{e}.gate"], params[f"e{e}.up"]], 0) for e in range(E)]).contiguous()
+        self.w_down = torch.stack([params[f"e{e}.down"] for e in range(E)]).contiguous()
+        self.router = Linear(params["router"])
+        self.correction = params["correction"].to(torch.float32).contiguous() if spec.corrected else None
+
+    def forward(self, x, batch):
+        spec = self.spec
+        logits = self.router.forward(x, out_dtype=torch.float32)
+        choice, weight = kernels.router_select(logits, self.correction, batch.positions, spec.top, spec.groups,
+                                               spec.groups_kept, spec.normalised, spec.weight_eps)
+        run = kernels.moe_grouped if kernels.moe_grouped_applies(x, x.shape[1], spec.intermediate_size) else kernels.moe_rows
+        return run(x, batch, None, self.w_gate_up, self.w_down, self.activation, choice=choice, weight=weight,
+                   identity=spec.identity)
+
+
+register_feed_forward("routed_experts", RoutedExperts)

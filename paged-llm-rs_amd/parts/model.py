@@ -16,7 +16,8 @@ from ..cache.layout import CacheLayout
 from ..config import load_config
 from ..errors import ConfigError, UnsupportedError, WeightError
 from ..weights.loader import ParamDecl, load_weights
-from . import attention, block, conv_attention, latent_attention, mlp, norm, parallel, recurrent, sink_attention, transforms  # noqa: F401  (register the built-in parts)
+from . import (attention, block, conv_attention, latent_attention, mlp, norm, parallel, recurrent, sink_attention,  # noqa: F401
+               tied_attention, transforms)                       # (register the built-in parts)
 from .linear import Linear, linears_of
 from .norm import PendingNorm
 from .registry import BLOCKS, EMBED_TRANSFORMS, FINAL_TRANSFORMS, LOGIT_TRANSFORMS, NORMS, lookup, prefixed, scoped
@@ -92,7 +93,7 @@ class LayerContext:
     the pages of the layer it reads from) and its state slots."""
 
     __slots__ = ("batch", "cache", "layer", "cache_layer", "writes_cache", "residual", "trace", "hand", "handed",
-                 "norm_after", "handed_out", "stream_rows")
+                 "norm_after", "handed_out", "stream_rows", "stream_addend")
 
     def __init__(self, batch, cache, layer: int, cache_layer: int, writes_cache: bool):
         # ``layer`` and ``cache_layer`` are the keys under which the cache keeps this run's state and the pages it
@@ -118,6 +119,10 @@ class LayerContext:
         # The rows of the stream in the model's type, where the part that last updated the stream left them
         # (a block that normalises sublayer outputs does; any block may read, replace or clear them).
         self.stream_rows = None
+        # Rows the decoder wants added to the 32-bit stream before this run (what the model began with, where the
+        # schedule says so), for a block that takes them into its own first pass (``takes_stream_addend``) and
+        # clears this; for any other block the decoder has added them already and this is None.
+        self.stream_addend = None
 
     def kv(self):
         return self.cache.layer_view(self.cache_layer, self.batch)
@@ -214,14 +219,32 @@ class DecoderModel:
         handed = None
         stream_rows = None
         schedule = self.spec.schedule
+        # (kept only where a run of the schedule adds it to the stream again)
+        began_with = resid.clone() if any(e.add_embedding for e in schedule) else None
         for at, entry in enumerate(schedule):
             own = entry.cache_from is None
             key = entry.layer if entry.cache_key is None else entry.cache_key
             ctx = LayerContext(batch, cache, key, key if own else entry.cache_from, own)
             if top is not None:
-                ctx.trace = top.child(self.spec.layers[entry.layer].weight_prefix)
+                # (a layer that runs again records under its prefix with ``.run<k>`` behind it, k = 1 for its second run)
+                again = sum(1 for e in schedule[:at] if e.layer == entry.layer)
+                prefix = self.spec.layers[entry.layer].weight_prefix
+                ctx.trace = top.child(prefix if again == 0 else f"{prefix}.run{again}")
             ctx.handed = handed
             ctx.stream_rows = stream_rows
+            if entry.add_embedding:
+                if getattr(self.blocks[entry.layer], "takes_stream_addend", False):
+                    ctx.stream_addend = began_with
+                else:
+                    # (a block that knows nothing of it gets a stream that holds every sum)
+                    if delta is not None:
+                        kernels.residual_add(resid, delta)
+                        delta = None
+                    if handed is not None and not isinstance(handed, kernels.HandedNorm):
+                        raise UnsupportedError("the layer before left work on the stream to this layer, which cannot take "
+                                               "what the model began with into the same pass")
+                    kernels.residual_add(resid, began_with)
+                    ctx.handed = ctx.stream_rows = None
             if at + 1 < len(schedule):
                 ctx.norm_after = getattr(self.blocks[schedule[at + 1].layer], "first_norm", None)
             delta = self.blocks[entry.layer].forward(resid, delta, ctx)

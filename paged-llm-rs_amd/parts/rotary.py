@@ -46,3 +46,28 @@ def rotary_tables(spec, device, shared: dict):
     if key not in shared:
         shared[key] = lookup(POSITIONS, spec.kind, "position encoding")(spec, device)
     return shared[key]
+
+
+def rotary_frequencies(dims: int, base: float, scaling=None, device=None) -> torch.Tensor:
+    """The frequencies base^(-2i/dims), i < dims / 2, worked out in 64-bit and rounded to 32-bit: for kernels that turn by
+    position * frequency without tables.  ``scaling`` = (factor, low, high, original) rescales them by their wavelength
+    l = 2 pi / f: kept where l < original / high, divided by ``factor`` where l > original / low, and between the two
+    (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
+    import math
+
+    if dims % 2 or dims <= 0:
+        raise UnsupportedError(f"a rotation over {dims} values, which do not pair")
+    out = []
+    for i in range(dims // 2):
+        f = float(base) ** (-2.0 * i / dims)
+        if scaling is not None:
+            factor, low, high, original = (float(v) for v in scaling)
+            length = 2.0 * math.pi / f
+            if low > 0 and length > original / low:
+                f = f / factor
+            elif length >= original / high:
+                s = (original / length - low) / (high - low)
+                f = (1.0 - s) * f / factor + s * f
+        out.append(f)
+    t = torch.tensor(out, dtype=torch.float64).to(torch.float32)
+    return t.to(device) if device is not None else t
