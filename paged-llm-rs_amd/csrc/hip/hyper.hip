@@ -422,16 +422,18 @@ extern "C" int pl_moe_sort(const int* ids, const int* src, const int* fed, const
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ slot_of,
                                                           float* __restrict__ out, int top, int W, int splits, size_t split_stride,
                                                           const float* __restrict__ weight, const int* __restrict__ choice,
-                                                          const void* __restrict__ x, int x_dtype, int E) {
+                                                          const void* __restrict__ x, int x_dtype, int E,
+                                                          const int* __restrict__ positions) {
     const int t = blockIdx.x;
     const float even = 1.f / static_cast<float>(top);
+    const bool padding = positions != nullptr && positions[t] < 0;        // (a row of padding has no identity expert either)
     for (int w = threadIdx.x * 4; w < W; w += blockDim.x * 4) {
         float4 sum = {0.f, 0.f, 0.f, 0.f};
         for (int c = 0; c < top; ++c) {
             const int slot = slot_of[t * top + c];
             const float share = weight != nullptr ? weight[t * top + c] : even;
             if (slot < 0) {
-                if (choice != nullptr && choice[t * top + c] >= E) {
+                if (choice != nullptr && !padding && choice[t * top + c] >= E) {
                     const size_t at = static_cast<size_t>(t) * W + w;
                     sum.x += load_as_float(x, x_dtype, at) * share;
                     sum.y += load_as_float(x, x_dtype, at + 1) * share;
@@ -459,13 +461,13 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
 
 extern "C" int pl_moe_combine(const float* y, const int* slot_of, float* out, int n, int top, int W, int splits,
                               long long split_stride, const float* weight, const int* choice, const void* x, int x_dtype,
-                              int E, hipStream_t stream) {
+                              int E, const int* positions, hipStream_t stream) {
     PL_REQUIRE(n >= 0 && top > 0 && W > 0 && W % 4 == 0 && splits >= 1, "moe_combine: %d rows of %d, %d a row, %d copies", n, W, top, splits);
     PL_REQUIRE(choice == nullptr || (x != nullptr && (x_dtype == PL_DTYPE_F32 || x_dtype == PL_DTYPE_BF16)),
                "moe_combine: identity experts need the rows they hand through");
     if (n == 0) return 0;
     moe_combine_kernel<<<n, 256, 0, stream>>>(y, slot_of, out, top, W, splits, static_cast<size_t>(split_stride), weight, choice,
-                                              x, x_dtype, E);
+                                              x, x_dtype, E, positions);
     PL_CHECK_LAUNCH("moe_combine");
     return 0;
 }

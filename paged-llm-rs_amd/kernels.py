@@ -80,7 +80,7 @@ def _signatures(lib) -> None:
         "pl_softcap": [p, f, ctypes.c_long, p],
         "pl_moe_rows": [p, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, p, p, i, p],
         "pl_moe_sort": [p, p, p, p, p, p, i, i, i, i, i, i, p, p, p, p],
-        "pl_moe_combine": [p, p, p, i, i, i, i, ctypes.c_longlong, p, p, p, i, i, p],
+        "pl_moe_combine": [p, p, p, i, i, i, i, ctypes.c_longlong, p, p, p, i, i, p, p],
         "pl_router_select": [p, i, p, p, i, i, i, i, i, i, f, p, p, p],
         "pl_wide_prepare": [p, p, i, i, i, f, p, p, p, i, p, p, p, i, i, i, p, p, p, i, i, i, i, i, i, p],
         "pl_parallel_step": [p, p, p, p, p, p, p, p, f, p, p, i, p, i, i, p],
@@ -1637,7 +1637,7 @@ def moe_grouped(x: torch.Tensor, batch, table, w_gate_up: torch.Tensor, w_down: 
     _check(lib.pl_gemm_tiled_grouped(hidden.data_ptr(), w_down.data_ptr(), y.data_ptr(), tile_group.data_ptr(), 0,
                                      W * F, tiles, slots, W, F, 3, 0, splits, stream))
     _check(lib.pl_moe_combine(y.data_ptr(), slot_of.data_ptr(), out.data_ptr(), n, top, W, splits, slots * W,
-                              _ptr(weight), _ptr(choice), x.data_ptr(), _code(x, "rows"), E, stream))
+                              _ptr(weight), _ptr(choice), x.data_ptr(), _code(x, "rows"), E, batch.positions.data_ptr(), stream))
     return out
 
 

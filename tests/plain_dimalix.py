@@ -197,7 +197,7 @@ def forward(config, w, tokens, streams=None):
     eps = config["norm"]["eps"]
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     positions = torch.arange(len(tokens))
-    first = w["embed"][tokens] * config["embedding"]["scale"]
+    first = w["embed"][tokens] * (config.get("embedding") or {}).get("scale", 1.0)
     x = first.clone()
     for i, again in layer_runs(config):
         layer = config["layers"][i]
