@@ -345,9 +345,40 @@ def mukenex_config(width: int, ff: int, heads: int, layers: int, vocab: int) -> 
             "logit_softcap": 30.0, "layers": [kinds[i % 3] for i in range(layers)]}
 
 
-DESIGNS = {"papivik": papivik_config, "lefavik": lefavik_config, "mukenex": mukenex_config}
+# --only dimalix: the Dimalix design (layers whose mixer and feed-forward read the same stream through a norm each and
+# join it with a gain a column; windowed attention over one small vector a token, and grouped attention inside chunks of
+# positions whose values are its keys, with one norm over all heads of q and of k and rescaled rotation frequencies; the
+# first layer of three with a dense feed-forward, the others with eight experts and two identity experts behind a router
+# that chooses two of them out of the better of two groups, each expert half the dense width; with six layers or more
+# the first three run twice, each further pass starting from the stream plus the embedding) at the same sizes, beside
+# Qwen3 dense and beside Mukenex, the design whose kernels are the nearest to these.
+def dimalix_config(width: int, ff: int, heads: int, layers: int, vocab: int) -> dict:
+    experts = {"kind": "moe", "expert": {"ff": ff // 2},
+               "router": {"experts": 8, "identity": 2, "top": 2, "groups": {"count": 2, "keep": 1}}}
+    kinds = [
+        {"type": "latent_attention", "mixer": {"heads": heads, "dim": 64, "rot_dim": 64, "vdim": 128, "kv_rank": 192,
+                                               "scale": 128 ** -0.5, "rot": {"dims": 64, "base": 1000000.0},
+                                               "mask": {"size": 512}}, "mlp": {"kind": "dense", "ff": ff}},
+        {"type": "attention", "mixer": {"heads": heads, "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                                        "rot": {"dims": 128, "base": 500000.0,
+                                                "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}},
+                                        "mask": {"size": 512}}, "mlp": experts},
+        {"type": "latent_attention", "mixer": {"heads": heads, "dim": 64, "rot_dim": 64, "vdim": 128, "kv_rank": 192,
+                                               "scale": 128 ** -0.5, "rot": {"dims": 64, "base": 1000000.0},
+                                               "mask": {"size": 512}}, "mlp": experts},
+    ]
+    config = {"architecture": "Dimalix", "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6}, "vocab": vocab, "width": width}
+    if layers >= 6:
+        config["layers"] = [kinds[i % 3] for i in range(layers - 3)]
+        config["loop"] = {"start": 0, "stop": 3, "times": 2}
+    else:
+        config["layers"] = [kinds[i % 3] for i in range(layers)]
+    return config
+
+
+DESIGNS = {"papivik": papivik_config, "lefavik": lefavik_config, "mukenex": mukenex_config, "dimalix": dimalix_config}
 # the models a design is measured beside, after Qwen3 dense
-BESIDE = {"mukenex": ("lefavik",)}
+BESIDE = {"mukenex": ("lefavik",), "dimalix": ("mukenex",)}
 
 
 def papivik_table(torch, args, design: str = "papivik") -> int:
@@ -478,8 +509,8 @@ def main() -> int:
     parser.add_argument("--ahead", choices=["on", "off"], default="on",
                         help="--only engine: whether the engine queues a decoding step before it has read the tokens "
                              "of the one before")
-    parser.add_argument("--size", choices=sorted(PAPIVIK_SIZES), default=None, help="--only papivik, lefavik or mukenex: one of the sizes alone")
-    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving", "products", "papivik", "lefavik", "mukenex"], default=None,
+    parser.add_argument("--size", choices=sorted(PAPIVIK_SIZES), default=None, help="--only papivik, lefavik, mukenex or dimalix: one of the sizes alone")
+    parser.add_argument("--only", choices=["decode", "prefill", "engine", "mixed", "serving", "products", "papivik", "lefavik", "mukenex", "dimalix"], default=None,
                         help="run one part alone: the decode steps at --batch, the prefill, or (not part of the "
                              "default line) the whole engine on 1/4/16/32/64/128 requests at once, 16 prompt tokens and "
                              "128 generated each, as the reference's own table of clients does; mixed: one step of a "
@@ -490,7 +521,7 @@ def main() -> int:
                              "by the library and by the two hand-written products of few rows; papivik: prefill and decode "
                              "of the Papivik design at layer sizes of the 0.6B and 8B shapes beside Qwen3 dense of the same "
                              "width, layers and vocabulary; lefavik: the same for the Lefavik design; mukenex: the same for the Mukenex "
-                             "design, beside Lefavik too")
+                             "design, beside Lefavik too; dimalix: the same for the Dimalix design, beside Mukenex too")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU; this engine has no multi-GPU path (N must be 1)")

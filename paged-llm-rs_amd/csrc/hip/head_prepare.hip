@@ -151,40 +151,64 @@ struct WidePrepareArgs {
     int H, G, D, Dp;
 };
 
-// A workgroup a token.  The row of q | k (with the biases) waits in LDS; two sums of squares over the whole
-// projections; then every value is normed, gained, turned and stored, heads in rows of Dp values with zeros behind.
+// A workgroup a token.  The row of q | k (with the biases) waits in LDS, each value times its gain (and the keys a
+// second time as they are: they are the values); two sums of squares over the whole projections; then a wave takes
+// a head at a time: normed, turned and stored, heads in rows of Dp values with zeros behind.  Every load from memory
+// stands before the first store, so none of them waits for one.
 template <typename T>
 __global__ __launch_bounds__(256) void wide_prepare_kernel(WidePrepareArgs a) {
-    extern __shared__ float wide_lds[];               // [H D + G D] values, [rot / 2] cosines, [rot / 2] sines
+    extern __shared__ float wide_lds[];               // [H D + G D] gained values, [G D] keys as projected, cosines, sines
     __shared__ float scratch[16];
     const int t = blockIdx.x;
     const int pos = a.positions[t];
     if (pos < 0) return;
     const int H = a.H, G = a.G, D = a.D, Dp = a.Dp, half = a.rot / 2;
     const int nq = H * D, nk = a.write_kv ? G * D : 0;
-    float* vals = wide_lds;
-    float* cs = wide_lds + H * D + G * D;
+    float* gained = wide_lds;
+    float* raw = wide_lds + (H + G) * D;
+    float* cs = raw + G * D;
     float* sn = cs + half;
     const float* src = a.rows + static_cast<size_t>(t) * a.stride + a.off;
     float ssq = 0.f, ssk = 0.f;
-    for (int e = threadIdx.x; e < nq + nk; e += blockDim.x) {
-        const float x = a.bias != nullptr ? src[e] + a.bias[e] : src[e];
-        vals[e] = x;
-        if (e < nq) ssq += x * x;
-        else ssk += x * x;
-    }
-    for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(static_cast<float>(pos) * a.freq[i], &sn[i], &cs[i]);
-    float inv_q = 1.f, inv_k = 1.f;
-    if (a.normed) {
-        ssq = block_sum(ssq, scratch);
-        inv_q = 1.f / sqrtf(ssq / static_cast<float>(nq) + a.eps);
-        if (nk > 0) {
-            ssk = block_sum(ssk, scratch);
-            inv_k = 1.f / sqrtf(ssk / static_cast<float>(nk) + a.eps);
+    if ((a.stride | a.off | nq | nk) % 4 == 0) {
+        for (int e = threadIdx.x * 4; e < nq + nk; e += blockDim.x * 4) {
+            float4 x = *reinterpret_cast<const float4*>(src + e);
+            if (a.bias != nullptr) {
+                const float4 b = *reinterpret_cast<const float4*>(a.bias + e);
+                x.x += b.x, x.y += b.y, x.z += b.z, x.w += b.w;
+            }
+            const float* gain = e < nq ? a.q_gain : a.k_gain;
+            float4 g = {1.f, 1.f, 1.f, 1.f};
+            if (gain != nullptr) g = *reinterpret_cast<const float4*>(gain + (e < nq ? e : e - nq));
+            const float ss = x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+            if (e < nq) {
+                ssq += ss;
+            } else {
+                ssk += ss;
+                *reinterpret_cast<float4*>(raw + e - nq) = x;
+            }
+            *reinterpret_cast<float4*>(gained + e) = make_float4(x.x * g.x, x.y * g.y, x.z * g.z, x.w * g.w);
+        }
+    } else {
+        for (int e = threadIdx.x; e < nq + nk; e += blockDim.x) {
+            const float x = a.bias != nullptr ? src[e] + a.bias[e] : src[e];
+            const float* gain = e < nq ? a.q_gain : a.k_gain;
+            const float g = gain != nullptr ? gain[e < nq ? e : e - nq] : 1.f;
+            if (e < nq) {
+                ssq += x * x;
+            } else {
+                ssk += x * x;
+                raw[e - nq] = x;
+            }
+            gained[e] = x * g;
         }
     }
-    __syncthreads();
-    T* q_dst = static_cast<T*>(a.q_out) + static_cast<size_t>(t) * H * Dp;
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        float s_i, c_i;
+        sincosf(static_cast<float>(pos) * a.freq[i], &s_i, &c_i);
+        cs[i] = c_i;
+        sn[i] = s_i;
+    }
     T* k_dst = nullptr;
     T* v_dst = nullptr;
     if (nk > 0) {
@@ -196,30 +220,36 @@ __global__ __launch_bounds__(256) void wide_prepare_kernel(WidePrepareArgs a) {
             v_dst = static_cast<T*>(a.v_pool) + row * G * Dp;
         }
     }
-    const int total = (H + (k_dst != nullptr ? G : 0)) * Dp;
-    for (int e = threadIdx.x; e < total; e += blockDim.x) {
-        const int head = e / Dp, d = e - head * Dp;
-        const bool query = head < H;
-        const int c = query ? head * D + d : nq + (head - H) * D + d;      // the value's place in `vals`
-        float x = 0.f, raw = 0.f;
-        if (d < D) {
-            const float inv = query ? inv_q : inv_k;
-            const float* gain = query ? a.q_gain : a.k_gain;
-            const int g0 = query ? 0 : nq;
-            raw = vals[c];
-            x = raw * inv * (gain != nullptr ? gain[c - g0] : 1.f);
-            if (d < a.rot) {
-                const int other = (d & 1) ? c - 1 : c + 1;
-                const float y = vals[other] * inv * (gain != nullptr ? gain[other - g0] : 1.f);
-                const int i = d >> 1;
-                x = (d & 1) ? x * cs[i] + y * sn[i] : x * cs[i] - y * sn[i];
-            }
+    float inv_q = 1.f, inv_k = 1.f;
+    if (a.normed) {
+        ssq = block_sum(ssq, scratch);
+        inv_q = 1.f / sqrtf(ssq / static_cast<float>(nq) + a.eps);
+        if (nk > 0) {
+            ssk = block_sum(ssk, scratch);
+            inv_k = 1.f / sqrtf(ssk / static_cast<float>(nk) + a.eps);
         }
-        if (query) {
-            q_dst[e] = from_float<T>(x);
-        } else {
-            k_dst[e - H * Dp] = from_float<T>(x);
-            v_dst[e - H * Dp] = from_float<T>(raw);
+    }
+    __syncthreads();
+    T* q_dst = static_cast<T*>(a.q_out) + static_cast<size_t>(t) * H * Dp;
+    const int lane = threadIdx.x % PL_WAVE, wave = threadIdx.x / PL_WAVE, waves = blockDim.x / PL_WAVE;
+    const int heads = H + (k_dst != nullptr ? G : 0);
+    for (int head = wave; head < heads; head += waves) {
+        const bool query = head < H;
+        const float inv = query ? inv_q : inv_k;
+        const float* mine = gained + head * D;                            // (the keys' heads follow the queries')
+        T* dst = query ? q_dst + head * Dp : k_dst + (head - H) * Dp;
+        for (int d = lane; d < Dp; d += PL_WAVE) {
+            float x = 0.f;
+            if (d < D) {
+                x = mine[d] * inv;
+                if (d < a.rot) {
+                    const float y = mine[(d & 1) ? d - 1 : d + 1] * inv;
+                    const int i = d >> 1;
+                    x = (d & 1) ? x * cs[i] + y * sn[i] : x * cs[i] - y * sn[i];
+                }
+            }
+            dst[d] = from_float<T>(x);
+            if (!query) v_dst[(head - H) * Dp + d] = from_float<T>(d < D ? raw[(head - H) * D + d] : 0.f);
         }
     }
 }
@@ -235,7 +265,7 @@ extern "C" int pl_wide_prepare(const float* rows, const float* bias, int stride,
                "wide_prepare: a rotation over %d values of a head of %d", rot, D);
     PL_REQUIRE(block_size > 0 && max_blocks > 0 && stride >= off + (H + G) * D, "wide_prepare: pages of %d, tables of %d, rows of %d values for %d from %d on",
                block_size, max_blocks, stride, (H + G) * D, off);
-    const size_t lds = (static_cast<size_t>(H + G) * D + rot) * sizeof(float);
+    const size_t lds = (static_cast<size_t>(H + 2 * G) * D + rot) * sizeof(float);
     PL_REQUIRE(lds <= 64 * 1024, "wide_prepare: %d + %d heads of %d are more than a workgroup's 64 KB hold", H, G, D);
     if (n == 0) return 0;
     WidePrepareArgs a{rows, bias, stride, off, normed, eps, q_gain, k_gain, freq, rot, positions, seq_of, block_table,

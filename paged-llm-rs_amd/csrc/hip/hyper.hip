@@ -493,12 +493,17 @@ __device__ __forceinline__ void wave_best(float& v, int& i) {
 // only members of the `kept` best groups can be chosen (the others count as minus infinity); the `top` largest are
 // chosen (the lower index among equals), in that order; a chosen output weighs s, divided, with `normalised`, by the
 // chosen ones' sum plus weight_eps.  Rows at position -1 choose nothing (-1, weight 0).
+// With `x` [n, W] and the router's matrix `w` [total, W] (both of type T) the wave works the logits out itself first,
+// 32-bit sums of the products in an order that W alone fixes: for steps of few rows, where a product's launch costs
+// more than the product.
+template <typename T>
 __global__ __launch_bounds__(64) void router_select_kernel(const float* __restrict__ z, int stride, const float* __restrict__ correction,
                                                            const int* __restrict__ positions, int total, int top, int groups,
                                                            int kept, int normalised, float weight_eps, int* __restrict__ choice,
-                                                           float* __restrict__ weight) {
+                                                           float* __restrict__ weight, const T* __restrict__ x,
+                                                           const T* __restrict__ w, int W) {
     extern __shared__ float router_lds[];             // score [total], choice score [total], group score [groups], kept or not [groups]
-    float* score = router_lds;
+    float* score = router_lds;                        // (and behind them, where the logits are worked out here: logits [total], the row [W])
     float* pick = router_lds + total;
     float* group = pick + total;
     float* stays = group + groups;
@@ -513,6 +518,18 @@ __global__ __launch_bounds__(64) void router_select_kernel(const float* __restri
         return;
     }
     const float* row = z + static_cast<size_t>(t) * stride;
+    if (x != nullptr) {
+        float* logits = stays + groups;
+        float* xs = logits + total;
+        for (int k = lane; k < W; k += PL_WAVE) xs[k] = to_float(x[static_cast<size_t>(t) * W + k]);
+        __syncthreads();
+        for (int e = 0; e < total; ++e) {
+            const float sum = moe_dot<T>(w + static_cast<size_t>(e) * W, xs, W, lane);
+            if (lane == 0) logits[e] = sum;
+        }
+        __syncthreads();
+        row = logits;
+    }
     float largest = -INFINITY;
     for (int e = lane; e < total; e += PL_WAVE) largest = fmaxf(largest, row[e]);
     largest = wave_max(largest);
@@ -585,17 +602,34 @@ __global__ __launch_bounds__(64) void router_select_kernel(const float* __restri
     }
 }
 
+// z [n, stride] holds the logits, or, where it is null, x [n, W] and w [total, W] of type `dtype` give them.
 extern "C" int pl_router_select(const float* z, int stride, const float* correction, const int* positions, int n, int total,
                                 int top, int groups, int kept, int normalised, float weight_eps, int* choice, float* weight,
-                                hipStream_t stream) {
-    PL_REQUIRE(n >= 0 && total > 0 && total <= 8192 && stride >= total && top > 0 && top <= total,
+                                const void* x, const void* w, int W, int dtype, hipStream_t stream) {
+    PL_REQUIRE(n >= 0 && total > 0 && total <= 8192 && top > 0 && top <= total && (z == nullptr || stride >= total),
                "router_select: %d rows, %d of %d outputs in rows of %d", n, top, total, stride);
+    PL_REQUIRE((z != nullptr) != (x != nullptr) && (x == nullptr || (w != nullptr && W > 0 && W <= 8192 && total <= 1024)),
+               "router_select: logits, or rows of up to 8192 and a router of up to 1024 outputs to work them out from");
     PL_REQUIRE(groups >= 1 && total % groups == 0 && kept >= 1 && kept <= groups && top <= kept * (total / groups),
                "router_select: %d outputs in %d groups of which %d are kept, %d chosen", total, groups, kept, top);
     if (n == 0) return 0;
-    const size_t lds = 2 * (static_cast<size_t>(total) + groups) * sizeof(float);
-    router_select_kernel<<<n, 64, lds, stream>>>(z, stride, correction, positions, total, top, groups, kept, normalised, weight_eps,
-                                                 choice, weight);
+    size_t lds = 2 * (static_cast<size_t>(total) + groups) * sizeof(float);
+    if (x == nullptr) {
+        router_select_kernel<float><<<n, 64, lds, stream>>>(z, stride, correction, positions, total, top, groups, kept, normalised,
+                                                            weight_eps, choice, weight, nullptr, nullptr, 0);
+    } else {
+        lds += (static_cast<size_t>(total) + W) * sizeof(float);
+        if (dtype == PL_DTYPE_F32)
+            router_select_kernel<float><<<n, 64, lds, stream>>>(nullptr, 0, correction, positions, total, top, groups, kept, normalised,
+                                                                weight_eps, choice, weight, static_cast<const float*>(x),
+                                                                static_cast<const float*>(w), W);
+        else if (dtype == PL_DTYPE_BF16)
+            router_select_kernel<bf16_t><<<n, 64, lds, stream>>>(nullptr, 0, correction, positions, total, top, groups, kept, normalised,
+                                                                 weight_eps, choice, weight, static_cast<const bf16_t*>(x),
+                                                                 static_cast<const bf16_t*>(w), W);
+        else
+            PL_REQUIRE(false, "router_select: dtype code %d", dtype);
+    }
     PL_CHECK_LAUNCH("router_select");
     return 0;
 }

@@ -81,7 +81,7 @@ def _signatures(lib) -> None:
         "pl_moe_rows": [p, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, p, p, i, p],
         "pl_moe_sort": [p, p, p, p, p, p, i, i, i, i, i, i, p, p, p, p],
         "pl_moe_combine": [p, p, p, i, i, i, i, ctypes.c_longlong, p, p, p, i, i, p, p],
-        "pl_router_select": [p, i, p, p, i, i, i, i, i, i, f, p, p, p],
+        "pl_router_select": [p, i, p, p, i, i, i, i, i, i, f, p, p, p, p, i, i, p],
         "pl_wide_prepare": [p, p, i, i, i, f, p, p, p, i, p, p, p, i, i, i, p, p, p, i, i, i, i, i, i, p],
         "pl_parallel_step": [p, p, p, p, p, p, p, p, f, p, p, i, p, i, i, p],
         "pl_gemm_tiled_grouped": [p, p, p, p, p, ctypes.c_longlong, i, i, i, i, i, i, i, p],
@@ -1641,27 +1641,47 @@ def moe_grouped(x: torch.Tensor, batch, table, w_gate_up: torch.Tensor, w_down: 
     return out
 
 
-def router_select(logits: torch.Tensor, correction, positions, top: int, groups: int = 1, kept: int = 1,
-                  normalised: bool = True, weight_eps: float = 1e-20):
+# A router's logits are worked out inside the kernel that chooses (one wave a row, the router's matrix from L2) for steps
+# of up to this many rows and routers of up to this many weights; beyond, a product of its own (the library's) is faster.
+ROUTER_FUSED_ROWS = 128
+ROUTER_FUSED_WEIGHTS = 1 << 18
+
+
+def router_fuses(rows: int, total: int, width: int) -> bool:
+    return rows <= ROUTER_FUSED_ROWS and total * width <= ROUTER_FUSED_WEIGHTS and width <= 8192 and total <= 1024
+
+
+def router_select(logits, correction, positions, top: int, groups: int = 1, kept: int = 1,
+                  normalised: bool = True, weight_eps: float = 1e-20, x=None, w=None):
     """A router's choice for every row of its 32-bit ``logits`` [n, outputs]: (chosen [n, top] int32, weights [n, top]
     32-bit).  Scores are the softmax over all outputs; the choice goes by score plus ``correction`` ([outputs] 32-bit, or
     None); outputs form ``groups`` equal groups of neighbours, a group counts by its best choice score, and only members
     of the best ``kept`` groups can be chosen; the ``top`` largest are chosen, the lower index among equals; a chosen
     output weighs its score, divided (``normalised``) by the chosen scores' sum plus ``weight_eps``.  Rows at
-    position -1 choose nothing (-1)."""
-    _need(logits, "router logits", None, torch.float32)
-    if logits.dim() != 2:
-        raise TensorError(f"router logits of shape {tuple(logits.shape)}")
-    n, total = logits.shape
+    position -1 choose nothing (-1).  With ``logits`` None the kernel works them out itself from the rows ``x`` [n, W]
+    and the router's matrix ``w`` [outputs, W] (one type; 32-bit sums)."""
+    if logits is not None:
+        _need(logits, "router logits", None, torch.float32)
+        if logits.dim() != 2:
+            raise TensorError(f"router logits of shape {tuple(logits.shape)}")
+        n, total = logits.shape
+        width, code, device = 0, F32, logits.device
+    else:
+        _need(x, "rows")
+        _need(w, "router matrix", None, x.dtype)
+        if x.dim() != 2 or w.dim() != 2 or w.shape[1] != x.shape[1]:
+            raise TensorError(f"rows of shape {tuple(x.shape)} for a router of shape {tuple(w.shape)}")
+        (n, width), total, code, device = x.shape, w.shape[0], _code(x, "rows"), x.device
     if correction is not None:
         _need(correction, "correction of the choice", (total,), torch.float32)
     if positions is not None:
         _need(positions, "positions", (n,), torch.int32)
-    choice = torch.empty((n, top), dtype=torch.int32, device=logits.device)
-    weight = torch.empty((n, top), dtype=torch.float32, device=logits.device)
-    _check(library().pl_router_select(logits.data_ptr(), total, _ptr(correction), _ptr(positions), n, total, int(top),
+    choice = torch.empty((n, top), dtype=torch.int32, device=device)
+    weight = torch.empty((n, top), dtype=torch.float32, device=device)
+    _check(library().pl_router_select(_ptr(logits), total, _ptr(correction), _ptr(positions), n, total, int(top),
                                       int(groups), int(kept), 1 if normalised else 0, float(weight_eps),
-                                      choice.data_ptr(), weight.data_ptr(), _stream()))
+                                      choice.data_ptr(), weight.data_ptr(), _ptr(x) if logits is None else 0,
+                                      _ptr(w) if logits is None else 0, int(width), code, _stream()))
     return choice, weight
 
 

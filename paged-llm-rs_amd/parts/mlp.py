@@ -194,9 +194,14 @@ class RoutedExperts:
 
     def forward(self, x, batch):
         spec = self.spec
-        logits = self.router.forward(x, out_dtype=torch.float32)
-        choice, weight = kernels.router_select(logits, self.correction, batch.positions, spec.top, spec.groups,
-                                               spec.groups_kept, spec.normalised, spec.weight_eps)
+        if kernels.router_fuses(x.shape[0], self.router.out_features, x.shape[1]):
+            # (few rows: the kernel that chooses works the logits out itself)
+            choice, weight = kernels.router_select(None, self.correction, batch.positions, spec.top, spec.groups, spec.groups_kept,
+                                                   spec.normalised, spec.weight_eps, x=x, w=self.router.weight)
+        else:
+            logits = self.router.forward(x, out_dtype=torch.float32)
+            choice, weight = kernels.router_select(logits, self.correction, batch.positions, spec.top, spec.groups,
+                                                   spec.groups_kept, spec.normalised, spec.weight_eps)
         run = kernels.moe_grouped if kernels.moe_grouped_applies(x, x.shape[1], spec.intermediate_size) else kernels.moe_rows
         return run(x, batch, None, self.w_gate_up, self.w_down, self.activation, choice=choice, weight=weight,
                    identity=spec.identity)

@@ -176,6 +176,29 @@ def test_a_routers_choice(total, top, groups, kept):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("total,top,groups,kept,width", [(10, 2, 2, 1, 256), (9, 3, 3, 2, 72), (64, 6, 8, 3, 1024), (4, 2, 1, 1, 100)])
+def test_a_router_that_works_its_logits_out_itself(dtype, total, top, groups, kept, width):
+    """The kernel that chooses, given rows and the router's matrix instead of logits, against the same kernel over logits
+    from 64-bit arithmetic: the same experts and weights but for close calls."""
+    from paged_llm_rs_amd import kernels
+
+    g = torch.Generator().manual_seed(total + width)
+    n = 120
+    assert kernels.router_fuses(n, total, width)
+    x = torch.randn((n, width), generator=g).to(dtype)
+    w = (torch.randn((total, width), generator=g) * 2.5 * width ** -0.5).to(dtype)
+    correction = (torch.randn((total,), generator=g) * 0.2).float()
+    positions = torch.arange(n, dtype=torch.int32)
+    positions[40] = -1
+    z = (x.double() @ w.double().T).float()
+    want_c, want_w = kernels.router_select(z.cuda(), correction.cuda(), positions.cuda(), top, groups, kept)
+    got_c, got_w = kernels.router_select(None, correction.cuda(), positions.cuda(), top, groups, kept, x=x.cuda(), w=w.cuda())
+    same = (got_c == want_c).all(-1).cpu()
+    assert int(same.sum()) >= n - 2 and bool(same[40]) and (got_c[40] == -1).all()
+    assert (got_w - want_w)[same.cuda()].abs().max() <= 2e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,rot,page", [(6, 2, 24, 10, 16), (4, 1, 16, 16, 4), (16, 1, 128, 128, 16), (3, 3, 40, 0, 8), (8, 2, 64, 32, 16),
                                             (2, 2, 22, 22, 16), (1, 1, 30, 2, 16)])
 def test_between_the_projections_and_the_attention_kernels_where_the_values_are_the_keys(dtype, H, G, D, rot, page):
@@ -187,9 +210,10 @@ def test_between_the_projections_and_the_attention_kernels_where_the_values_are_
     from paged_llm_rs_amd.cache.pools import LayerKV
 
     g = torch.Generator().manual_seed(H * 100 + D)
-    n, off, eps = 23, 3, 1e-5
+    n, eps = 23, 1e-5
+    off, behind = (4, 8) if D % 8 == 0 else (3, 5)       # (rows that the kernel reads four values at a time, and rows it cannot)
     padded = D if dtype == torch.float32 else (D + 15) // 16 * 16
-    rows = torch.randn((n, off + (H + G) * D + 5), generator=g, dtype=torch.float64)
+    rows = torch.randn((n, off + (H + G) * D + behind), generator=g, dtype=torch.float64)
     bias = torch.randn(((H + G) * D,), generator=g, dtype=torch.float64)
     q_gain = 1 + 0.3 * torch.randn((H * D,), generator=g, dtype=torch.float64)
     k_gain = 1 + 0.3 * torch.randn((G * D,), generator=g, dtype=torch.float64)
