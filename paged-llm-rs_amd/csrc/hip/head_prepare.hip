@@ -266,13 +266,20 @@ extern "C" int pl_wide_prepare(const float* rows, const float* bias, int stride,
     PL_REQUIRE(block_size > 0 && max_blocks > 0 && stride >= off + (H + G) * D, "wide_prepare: pages of %d, tables of %d, rows of %d values for %d from %d on",
                block_size, max_blocks, stride, (H + G) * D, off);
     const size_t lds = (static_cast<size_t>(H + 2 * G) * D + rot) * sizeof(float);
-    PL_REQUIRE(lds <= 64 * 1024, "wide_prepare: %d + %d heads of %d are more than a workgroup's 64 KB hold", H, G, D);
+    PL_REQUIRE(lds <= 160 * 1024 - 256, "wide_prepare: %d + %d heads of %d are more than a workgroup's LDS holds", H, G, D);
+    PL_REQUIRE(dtype == PL_DTYPE_F32 || dtype == PL_DTYPE_BF16, "wide_prepare: dtype code %d", dtype);
     if (n == 0) return 0;
     WidePrepareArgs a{rows, bias, stride, off, normed, eps, q_gain, k_gain, freq, rot, positions, seq_of, block_table,
                       max_blocks, block_size, write_kv, q_out, k_pool, v_pool, H, G, D, Dp};
+    if (lds > 48 * 1024) {
+        // (a launch that asks for more than 48 KB says so first)
+        const void* kernel = dtype == PL_DTYPE_F32 ? reinterpret_cast<const void*>(&wide_prepare_kernel<float>)
+                                                   : reinterpret_cast<const void*>(&wide_prepare_kernel<bf16_t>);
+        const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+        PL_REQUIRE(e == hipSuccess, "wide_prepare: %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    }
     if (dtype == PL_DTYPE_F32) wide_prepare_kernel<float><<<n, 256, lds, stream>>>(a);
-    else if (dtype == PL_DTYPE_BF16) wide_prepare_kernel<bf16_t><<<n, 256, lds, stream>>>(a);
-    else PL_REQUIRE(false, "wide_prepare: dtype code %d", dtype);
+    else wide_prepare_kernel<bf16_t><<<n, 256, lds, stream>>>(a);
     PL_CHECK_LAUNCH("wide_prepare");
     return 0;
 }

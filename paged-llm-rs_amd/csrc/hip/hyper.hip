@@ -488,30 +488,67 @@ __device__ __forceinline__ void wave_best(float& v, int& i) {
     }
 }
 
-// A wave a row.  z [n, stride] are the router's 32-bit logits over `total` outputs.  s = softmax(z); the choice goes
+// Four dot products of a wave at once, rows e0, e0 + step, ... of w with a row of 32-bit values in LDS, so that the
+// loads of all four are on their way together; every lane gets the sums.  A row at or beyond `total` gives 0.
+template <typename T>
+__device__ __forceinline__ void router_dots(const T* __restrict__ w, const float* xs, int K, int lane, int e0, int step, int total,
+                                            float (&out)[4]) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    const T* rows[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) rows[j] = w + static_cast<size_t>(e0 + j * step < total ? e0 + j * step : e0) * K;
+    if (sizeof(T) == 2 && K % 8 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0) {
+        for (int k = lane * 8; k < K; k += 64 * 8) {
+            uint4 raw[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) raw[j] = *reinterpret_cast<const uint4*>(rows[j] + k);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t word[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[j] = fmaf(__uint_as_float(word[i] << 16), xs[k + 2 * i], acc[j]);
+                    acc[j] = fmaf(__uint_as_float(word[i] & 0xffff0000u), xs[k + 2 * i + 1], acc[j]);
+                }
+            }
+        }
+    } else {
+        for (int k = lane; k < K; k += 64) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = fmaf(to_float(rows[j][k]), xs[k], acc[j]);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[j] = wave_sum(acc[j]);
+}
+
+// A workgroup a row; its first wave chooses.  z [n, stride] are the router's 32-bit logits over `total` outputs.
+// s = softmax(z); the choice goes
 // by s + correction; outputs form `groups` equal groups of neighbours, a group counts by its largest choice score and
 // only members of the `kept` best groups can be chosen (the others count as minus infinity); the `top` largest are
 // chosen (the lower index among equals), in that order; a chosen output weighs s, divided, with `normalised`, by the
 // chosen ones' sum plus weight_eps.  Rows at position -1 choose nothing (-1, weight 0).
-// With `x` [n, W] and the router's matrix `w` [total, W] (both of type T) the wave works the logits out itself first,
-// 32-bit sums of the products in an order that W alone fixes: for steps of few rows, where a product's launch costs
-// more than the product.
+// With `x` [n, W] and the router's matrix `w` [total, W] (both of type T) the workgroup works the logits out itself
+// first, all its waves at it, 32-bit sums of the products in an order that W alone fixes: for steps of few rows, where
+// a product's launch costs more than the product.  (The waves behind the first then walk through the choice with
+// nothing to do, so that every barrier is met by all.)
 template <typename T>
-__global__ __launch_bounds__(64) void router_select_kernel(const float* __restrict__ z, int stride, const float* __restrict__ correction,
-                                                           const int* __restrict__ positions, int total, int top, int groups,
-                                                           int kept, int normalised, float weight_eps, int* __restrict__ choice,
-                                                           float* __restrict__ weight, const T* __restrict__ x,
-                                                           const T* __restrict__ w, int W) {
+__global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ z, int stride, const float* __restrict__ correction,
+                                                            const int* __restrict__ positions, int total_all, int top, int groups_all,
+                                                            int kept, int normalised, float weight_eps, int* __restrict__ choice,
+                                                            float* __restrict__ weight, const T* __restrict__ x,
+                                                            const T* __restrict__ w, int W) {
     extern __shared__ float router_lds[];             // score [total], choice score [total], group score [groups], kept or not [groups]
     float* score = router_lds;                        // (and behind them, where the logits are worked out here: logits [total], the row [W])
-    float* pick = router_lds + total;
-    float* group = pick + total;
-    float* stays = group + groups;
-    const int t = blockIdx.x, lane = threadIdx.x;
+    float* pick = router_lds + total_all;
+    float* group = pick + total_all;
+    float* stays = group + groups_all;
+    const int t = blockIdx.x, lane = threadIdx.x % PL_WAVE, wave = threadIdx.x / PL_WAVE, waves = blockDim.x / PL_WAVE;
+    const bool chooser = wave == 0;
     int* chosen = choice + static_cast<size_t>(t) * top;
     float* counts = weight + static_cast<size_t>(t) * top;
     if (positions != nullptr && positions[t] < 0) {
-        for (int c = lane; c < top; c += PL_WAVE) {
+        for (int c = threadIdx.x; c < top; c += blockDim.x) {
             chosen[c] = -1;
             counts[c] = 0.f;
         }
@@ -519,25 +556,30 @@ __global__ __launch_bounds__(64) void router_select_kernel(const float* __restri
     }
     const float* row = z + static_cast<size_t>(t) * stride;
     if (x != nullptr) {
-        float* logits = stays + groups;
-        float* xs = logits + total;
-        for (int k = lane; k < W; k += PL_WAVE) xs[k] = to_float(x[static_cast<size_t>(t) * W + k]);
+        float* logits = stays + groups_all;
+        float* xs = logits + total_all;
+        for (int k = threadIdx.x; k < W; k += blockDim.x) xs[k] = to_float(x[static_cast<size_t>(t) * W + k]);
         __syncthreads();
-        for (int e = 0; e < total; ++e) {
-            const float sum = moe_dot<T>(w + static_cast<size_t>(e) * W, xs, W, lane);
-            if (lane == 0) logits[e] = sum;
+        for (int e0 = wave; e0 < total_all; e0 += 4 * waves) {
+            float sums[4];
+            router_dots<T>(w, xs, W, lane, e0, waves, total_all, sums);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (lane == 0 && e0 + j * waves < total_all) logits[e0 + j * waves] = sums[j];
         }
         __syncthreads();
         row = logits;
     }
+    // (a wave that does not choose sees no outputs and no groups)
+    const int total = chooser ? total_all : 0, groups = chooser ? groups_all : 0;
     float largest = -INFINITY;
     for (int e = lane; e < total; e += PL_WAVE) largest = fmaxf(largest, row[e]);
     largest = wave_max(largest);
     float sum = 0.f;
     for (int e = lane; e < total; e += PL_WAVE) {
-        const float x = expf(row[e] - largest);
-        score[e] = x;
-        sum += x;
+        const float v = expf(row[e] - largest);
+        score[e] = v;
+        sum += v;
     }
     sum = wave_sum(sum);
     for (int e = lane; e < total; e += PL_WAVE) {
@@ -546,29 +588,28 @@ __global__ __launch_bounds__(64) void router_select_kernel(const float* __restri
         pick[e] = correction != nullptr ? s + correction[e] : s;
     }
     __syncthreads();
-    if (groups > 1) {
-        const int size = total / groups;
+    if (groups_all > 1) {
+        const int size = total_all / groups_all;
         for (int g = lane; g < groups; g += PL_WAVE) {
             float best = -INFINITY;
             for (int e = g * size; e < (g + 1) * size; ++e) best = fmaxf(best, pick[e]);
             group[g] = best;
+            stays[g] = 0.f;
         }
         __syncthreads();
         // the best `kept` groups keep their members, the others' members leave
-        for (int g = lane; g < groups; g += PL_WAVE) stays[g] = 0.f;
-        __syncthreads();
         for (int k = 0; k < kept; ++k) {
             float v = -INFINITY;
             int at = 0x7fffffff;
             for (int g = lane; g < groups; g += PL_WAVE) {
-                const float x = group[g];
-                if (stays[g] == 0.f && (at == 0x7fffffff || x > v)) {
-                    v = x;
+                const float s = group[g];
+                if (stays[g] == 0.f && (at == 0x7fffffff || s > v)) {
+                    v = s;
                     at = g;
                 }
             }
             wave_best(v, at);
-            if (lane == 0 && at != 0x7fffffff) stays[at] = 1.f;
+            if (chooser && lane == 0 && at != 0x7fffffff) stays[at] = 1.f;
             __syncthreads();
         }
         for (int e = lane; e < total; e += PL_WAVE)
@@ -580,24 +621,24 @@ __global__ __launch_bounds__(64) void router_select_kernel(const float* __restri
         float v = -INFINITY;
         int at = 0x7fffffff;
         for (int e = lane; e < total; e += PL_WAVE) {
-            const float x = pick[e];
-            if (!isnan(x) && (x > v || (x == v && e < at))) {
-                v = x;
+            const float s = pick[e];
+            if (!isnan(s) && (s > v || (s == v && e < at))) {
+                v = s;
                 at = e;
             }
         }
         wave_best(v, at);
         if (at == 0x7fffffff) at = -1;               // (nothing left to choose from)
-        const float s = at >= 0 ? score[at] : 0.f;
+        const float s = (chooser && at >= 0) ? score[at] : 0.f;
         chosen_sum += s;
-        if (lane == 0) {
+        if (chooser && lane == 0) {
             chosen[c] = at;
             counts[c] = s;
             if (at >= 0) pick[at] = NAN;             // (taken: below every other value, minus infinity included)
         }
         __syncthreads();
     }
-    if (normalised) {
+    if (normalised && chooser) {
         for (int c = lane; c < top; c += PL_WAVE) counts[c] = counts[c] / (chosen_sum + weight_eps);
     }
 }
@@ -620,11 +661,11 @@ extern "C" int pl_router_select(const float* z, int stride, const float* correct
     } else {
         lds += (static_cast<size_t>(total) + W) * sizeof(float);
         if (dtype == PL_DTYPE_F32)
-            router_select_kernel<float><<<n, 64, lds, stream>>>(nullptr, 0, correction, positions, total, top, groups, kept, normalised,
+            router_select_kernel<float><<<n, 256, lds, stream>>>(nullptr, 0, correction, positions, total, top, groups, kept, normalised,
                                                                 weight_eps, choice, weight, static_cast<const float*>(x),
                                                                 static_cast<const float*>(w), W);
         else if (dtype == PL_DTYPE_BF16)
-            router_select_kernel<bf16_t><<<n, 64, lds, stream>>>(nullptr, 0, correction, positions, total, top, groups, kept, normalised,
+            router_select_kernel<bf16_t><<<n, 256, lds, stream>>>(nullptr, 0, correction, positions, total, top, groups, kept, normalised,
                                                                  weight_eps, choice, weight, static_cast<const bf16_t*>(x),
                                                                  static_cast<const bf16_t*>(w), W);
         else

@@ -200,12 +200,12 @@ def test_a_router_that_works_its_logits_out_itself(dtype, total, top, groups, ke
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,D,rot,page", [(6, 2, 24, 10, 16), (4, 1, 16, 16, 4), (16, 1, 128, 128, 16), (3, 3, 40, 0, 8), (8, 2, 64, 32, 16),
-                                            (2, 2, 22, 22, 16), (1, 1, 30, 2, 16)])
+                                            (2, 2, 22, 22, 16), (1, 1, 30, 2, 16), (64, 32, 128, 64, 16)])
 def test_between_the_projections_and_the_attention_kernels_where_the_values_are_the_keys(dtype, H, G, D, rot, page):
     """Queries out, keys and values into scattered pages, against 64-bit arithmetic: the biases first, one statistic
     over all heads of q and one over all heads of k, a gain a column, the first values of every head turned in pairs,
     heads in padded rows with zeros behind them, the values the keys as they were before norm and rotation; rows of
-    padding write nothing."""
+    padding write nothing.  (The last case's rows take more of a workgroup's LDS than a launch gets unasked.)"""
     from paged_llm_rs_amd import kernels
     from paged_llm_rs_amd.cache.pools import LayerKV
 
