@@ -348,13 +348,13 @@ def mukenex_config(width: int, ff: int, heads: int, layers: int, vocab: int) -> 
 # --only dimalix: the Dimalix design (layers whose mixer and feed-forward read the same stream through a norm each and
 # join it with a gain a column; windowed attention over one small vector a token, and grouped attention inside chunks of
 # positions whose values are its keys, with one norm over all heads of q and of k and rescaled rotation frequencies; the
-# first layer of three with a dense feed-forward, the others with eight experts and two identity experts behind a router
-# that chooses two of them out of the better of two groups, each expert half the dense width; with six layers or more
+# first layer of three with a dense feed-forward, the others with eight experts and four identity experts behind a router
+# that chooses two of them out of the better two of four groups, each expert half the dense width; with six layers or more
 # the first three run twice, each further pass starting from the stream plus the embedding) at the same sizes, beside
 # Qwen3 dense and beside Mukenex, the design whose kernels are the nearest to these.
 def dimalix_config(width: int, ff: int, heads: int, layers: int, vocab: int) -> dict:
     experts = {"kind": "moe", "expert": {"ff": ff // 2},
-               "router": {"experts": 8, "identity": 2, "top": 2, "groups": {"count": 2, "keep": 1}}}
+               "router": {"experts": 8, "identity": 4, "top": 2, "groups": {"count": 4, "keep": 2}}}
     kinds = [
         {"type": "latent_attention", "mixer": {"heads": heads, "dim": 64, "rot_dim": 64, "vdim": 128, "kv_rank": 192,
                                                "scale": 128 ** -0.5, "rot": {"dims": 64, "base": 1000000.0},

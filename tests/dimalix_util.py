@@ -22,9 +22,11 @@ def attention(heads, kv_heads, dim, scale, chunk=None, turned=None, base=10000.0
     return {"type": "attention", "mixer": m, "mlp": mlp}
 
 
-def latent(heads, dim, rot_dim, vdim, kv_rank, scale, base=10000.0, window=None, mlp=None):
+def latent(heads, dim, rot_dim, vdim, kv_rank, scale, base=10000.0, window=None, scaling=None, mlp=None):
     m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "scale": scale,
          "rot": {"dims": rot_dim, "base": base}}
+    if scaling is not None:
+        m["rot"]["scaling"] = dict(zip(("factor", "low", "high", "original"), scaling))
     if window is not None:
         m["mask"] = {"size": window}
     return {"type": "latent_attention", "mixer": m, "mlp": mlp}
@@ -79,7 +81,7 @@ ONES = model(100, 97, [
 # width that the grouped products on the matrix cores take.
 PLAIN = model(256, 300, [
     latent(8, 64, 64, 64, 192, 0.09, base=10000.0, mlp=moe(8, 2, 64)),
-    attention(16, 1, 128, 0.1, mlp=dense(320)),
+    attention(16, 1, 128, 0.1, mlp=dense(352)),
     attention(4, 2, 64, 0.15, chunk=64, turned=32, scaling=(8.0, 1.0, 4.0, 2048), mlp=moe(8, 4, 128, identity=2, groups=(5, 3))),
     latent(2, 128, 64, 128, 192, 0.07, base=10000.0, window=64, mlp=dense(256)),
     attention(8, 8, 32, 0.2, chunk=100, mlp=moe(16, 3, 64, identity=4, groups=(4, 2))),

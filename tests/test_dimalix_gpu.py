@@ -148,7 +148,7 @@ def _route64(z, correction, top, groups, kept):
     return chosen, weight / (weight.sum(-1, keepdim=True) + 1e-20)
 
 
-@pytest.mark.parametrize("total,top,groups,kept", [(10, 2, 2, 1), (9, 2, 3, 2), (1, 1, 1, 1), (4, 4, 4, 4), (64, 6, 8, 3), (256, 8, 8, 4),
+@pytest.mark.parametrize("total,top,groups,kept", [(12, 2, 3, 1), (9, 2, 3, 2), (1, 1, 1, 1), (4, 4, 4, 4), (64, 6, 8, 3), (256, 8, 8, 4),
                                                    (300, 5, 1, 1), (6, 3, 2, 1), (5, 3, 1, 1), (128, 1, 128, 1)])
 def test_a_routers_choice(total, top, groups, kept):
     """Chosen experts, their order and weights against 64-bit arithmetic over the same 32-bit logits, with a correction
@@ -176,7 +176,7 @@ def test_a_routers_choice(total, top, groups, kept):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("total,top,groups,kept,width", [(10, 2, 2, 1, 256), (9, 3, 3, 2, 72), (64, 6, 8, 3, 1024), (4, 2, 1, 1, 100)])
+@pytest.mark.parametrize("total,top,groups,kept,width", [(12, 3, 3, 1, 320), (9, 3, 3, 2, 72), (64, 6, 8, 3, 1024), (4, 2, 1, 1, 100)])
 def test_a_router_that_works_its_logits_out_itself(dtype, total, top, groups, kept, width):
     """The kernel that chooses, given rows and the router's matrix instead of logits, against the same kernel over logits
     from 64-bit arithmetic: the same experts and weights but for close calls."""
@@ -329,6 +329,7 @@ def test_experts_behind_a_router(dtype, experts, identity, top, ff, width, rows)
 ALONE = {
     "latent, a window": [du.latent(3, 24, 8, 40, 56, 0.3, base=300.0, window=11)],
     "latent, no window": [du.latent(2, 16, 12, 16, 20, 0.4, base=40.0)],
+    "latent, rescaled frequencies": [du.latent(2, 16, 12, 16, 20, 0.4, base=40.0, window=30, scaling=(5.0, 1.0, 2.0, 30))],
     "attention, chunks of 7, part of a head turns, rescaled frequencies": [du.attention(6, 3, 24, 0.4, chunk=7, turned=14, base=60.0,
                                                                                          scaling=(4.0, 1.0, 3.0, 40))],
     "attention, no mask": [du.attention(2, 1, 40, 0.2, base=500.0)],
