@@ -857,6 +857,70 @@ def test_a_layer_that_runs_twice_and_layers_that_read_another_layers_cache(tmp_p
         assert worst <= tolerance, f"{worst:.3e} at {where}"
 
 
+# --- a stretch of layers that starts again from the stream plus what the model began with ------------------------------------
+
+class AgainConfig(SharingConfig):
+    """Two pre-norm layers run as 0, 1, 0, 1, the second pass with pages of its own and behind x + embedding."""
+
+    def model_spec(self):
+        from paged_llm_rs_amd.config import ScheduleEntry
+
+        spec = super().model_spec()
+        schedule = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0, cache_key=3, add_embedding=True), ScheduleEntry(1, cache_key=4))
+        return type(spec)(**{**spec.__dict__, "layers": spec.layers[:2], "schedule": schedule})
+
+
+AGAIN = dict(SHARING, architectures=["AgainToyForCausalLM"], model_type="again_toy")
+
+
+def again_plain(weights, tokens):
+    cfg = AGAIN
+    w = {k: v.double() for k, v in weights.items()}
+    n, eps = len(tokens), cfg["rms_norm_eps"]
+    nq, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    positions = torch.arange(n)
+    first = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+    x = first.clone()
+    for layer, again in ((0, False), (1, False), (0, True), (1, False)):
+        p = f"model.layers.{layer}"
+        if again:
+            x = x + first
+        h = plain.rms_norm(x, w[f"{p}.input_layernorm.weight"], eps)
+        q = plain.apply_rope(plain.rms_norm((h @ w[f"{p}.self_attn.q_proj.weight"].T).reshape(n, nq, d), w[f"{p}.self_attn.q_norm.weight"], eps),
+                             positions, cfg["rope_theta"])
+        k = plain.apply_rope(plain.rms_norm((h @ w[f"{p}.self_attn.k_proj.weight"].T).reshape(n, nkv, d), w[f"{p}.self_attn.k_norm.weight"], eps),
+                             positions, cfg["rope_theta"])
+        v = (h @ w[f"{p}.self_attn.v_proj.weight"].T).reshape(n, nkv, d)
+        out = plain.attention_core(q, plain.repeat_kv(k, nq // nkv), plain.repeat_kv(v, nq // nkv), 1.0 / math.sqrt(d))
+        x = x + out.reshape(n, nq * d) @ w[f"{p}.self_attn.o_proj.weight"].T
+        x = x + plain.swiglu_mlp(plain.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], eps), w, f"{p}.mlp")
+    return plain.rms_norm(x, w["model.norm.weight"], eps) @ w["model.embed_tokens.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_stretch_that_starts_again_from_the_stream_plus_the_embedding(tmp_path, dtype):
+    """`ScheduleEntry(add_embedding=True)` in front of a block that knows nothing of it: the decoder adds what the layer
+    before left unadded, then what the model began with; every schedule of replay agrees with the plain implementation."""
+    from safetensors.torch import load_file
+
+    from paged_llm_rs_amd import register_architecture, write_random_model
+    from paged_llm_rs_amd.engine.replay import Replayer
+
+    register_architecture("AgainToyForCausalLM", AgainConfig, model_type="again_toy")
+    folder = write_random_model(tmp_path / "again", AGAIN, seed=22, std=0.15, gain_std=0.2, dtype=dtype)
+    weights = load_file(str(folder / "model.safetensors"))
+    prompts = ru.make_prompts(AGAIN["vocab_size"], [50, 13, 77, 34], seed=9)
+    want = {name: again_plain(weights, toks) for name, toks in prompts.items()}
+    tolerance = 1e-5 if dtype == "float32" else 3e-2      # (four runs of layers whose stream grows by the embedding)
+    for steps, live in ((ru.whole(prompts), 1), (ru.tail_decoded(prompts, 20), 1), (ru.portions(prompts), 1),
+                        (ru.mixed(prompts, seed=5, max_live=3), 3)):
+        r = Replayer(folder, dtype, max_tokens=ru.pool_tokens(prompts, live), block_size=8, max_live=4)
+        assert [g.layers for g in r.cache.layout.groups] == [[0, 1, 3, 4]], "every run owns pages"
+        got = ru.collect(r, steps)
+        worst, where = ru.worst_error(got, want)
+        assert worst <= tolerance, f"{worst:.3e} at {where}"
+
+
 # --- a toy norm and a toy arrangement of a layer ----------------------------------------------------------------------------
 
 class CenteredNorm:
